@@ -91,3 +91,4 @@ def _ensure_builtin() -> None:
     from ..parts import llama4 as _llama4  # noqa: F401
     from ..parts import rovidra as _rovidra  # noqa: F401
     from ..parts import tiradra as _tiradra  # noqa: F401
+    from ..parts import mazotar as _mazotar  # noqa: F401

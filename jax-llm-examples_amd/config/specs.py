@@ -82,6 +82,8 @@ class ModelPlan:
     head: PartSpec | None = None
     # what is done to the residual stream where a run of the order ``enters_pass`` (see parts/loop.py); None: no loop
     loop: PartSpec | None = None
+    # the kind of residual stream the layers work on (see parts/residual.py); None: one stream, branch outputs added
+    residual: PartSpec | None = None
 
     def __post_init__(self) -> None:
         seen_write: dict[int, int] = {}

@@ -7,7 +7,7 @@ import torch
 
 from ..config.registry import architecture_name, get_architecture, read_config_json
 from ..parts.model import DecoderModel
-from ..weights.loader import load_weights
+from ..weights.loader import checkpoint_shapes, load_weights
 from ..weights.random_init import init_random_
 
 _DTYPES = {
@@ -60,6 +60,8 @@ def load_model(model_dir, dtype="bfloat16", device="cuda:0") -> DecoderModel:
     top = read_config_json(model_dir)
     arch = get_architecture(architecture_name(top))
     cfg = arch.parse_config(top)
+    if hasattr(arch, "complete_config"):  # (sizes that the file leaves to the tensors' shapes)
+        cfg = arch.complete_config(cfg, checkpoint_shapes(model_dir, getattr(arch, "optional_prefixes", ())))
     model = build_model(arch, cfg, dtype, device)
     model.allocate()
     load_weights(model, os.fspath(model_dir), arch.bindings(cfg, model.plan),

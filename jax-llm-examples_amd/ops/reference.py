@@ -49,6 +49,77 @@ class ReferenceOps:
         row = torch.where(prev < 0, torch.full_like(tok, buckets), (prev * mul_prev + tok * mul_cur) % buckets)
         return table[tok].float() + pair_table[row].float()
 
+    def embed_sinusoid(self, token_ids, positions, table, multiplier: float, rates):
+        """``table[token] * multiplier`` plus the position's sinusoid: entry ``2i`` is ``sin(pos * rates[i])``, entry
+        ``2i + 1`` the cosine (``rates``: float32 ``[ceil(hidden / 2)]``; the angle a float32 product); float32."""
+        x = table[token_ids.long()].float() * float(multiplier)
+        d = x.shape[1]
+        ang = positions.float()[:, None] * rates.float()[None, :]
+        wave = torch.stack([torch.sin(ang), torch.cos(ang)], dim=-1).reshape(x.shape[0], -1)
+        return x + wave[:, :d]
+
+    # ------------------------------------------------------------------ several residual streams
+    def streams_mix_norm(self, xs, update, inw, weight, eps: float, out_dtype, want32: bool = False, norm: bool = True):
+        """``xs``: float32 ``[N, S, D]``, changed in place.  With ``update`` (a branch output ``y`` ``[N, D]``, ``mix``
+        ``[S, S]`` indexed ``[from, to]``, ``outw`` ``[S]``): ``X_t <- sum_s mix[s, t] X_s + outw[t] y`` for all ``t``
+        at once.  Then (``norm``) ``u = sum_s inw[s] X_s`` (``inw`` ``None``: the plain sum) and ``h = u /
+        sqrt(mean(u^2) + eps) * weight``.  Returns ``(h in out_dtype, h in float32 or None)``."""
+        if update is not None:
+            y = self.materialize(update.y).float()
+            new = torch.einsum("st,nsd->ntd", update.mix.float(), xs) + update.outw.float()[None, :, None] * y[:, None, :]
+            xs.copy_(new)
+        if not norm:
+            return None, None
+        u = xs.sum(dim=1) if inw is None else torch.einsum("s,nsd->nd", inw.float(), xs)
+        h = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+        if weight is not None:
+            h = h * weight.float()
+        return h.to(out_dtype), (h if want32 else None)
+
+    # ------------------------------------------------------------------ a matrix memory per head
+    def mlstm(self, rows, gates, b_gates, norm_weight, num_heads: int, head_dim: int, value_dim: int, cap: float,
+              eps: float, floor: float, state, ctx):
+        """``rows``: ``[N, 2 H dk + 2 H dv]`` = q | k | v | output gate in the run dtype; ``gates``: float32 ``[N, 2 H]``
+        = the input gates' and the forget gates' pre-activations without their biases ``b_gates``.  Per head, token
+        by token from the request's state (``state[slot, phase]``: ``[H, dk dv + dk + 1]`` = C, n, m; the new state
+        goes to ``state[slot, 1 - phase]``)::
+
+            i = cap tanh((a + b_i) / cap);  f = logsigmoid(cap tanh((b + b_f) / cap));  m' = max(f + m, i)
+            C' = exp(f + m - m') C + exp(i - m') k v^T;  n' likewise with k;  o = C'^T q / (max(|n' . q|, exp(-m')) + floor)
+
+        with ``q`` times ``dk^(-1/2)``; then every head's ``o`` divided by its root mean square (``eps``), times
+        ``norm_weight``, times the sigmoid of the output gate.  ``[N, H dv]`` in the run dtype."""
+        n = rows.shape[0]
+        H, dk, dv = num_heads, head_dim, value_dim
+        r = rows.float()
+        q = r[:, : H * dk].reshape(n, H, dk) * (dk ** -0.5)
+        k = r[:, H * dk: 2 * H * dk].reshape(n, H, dk)
+        v = r[:, 2 * H * dk: 2 * H * dk + H * dv].reshape(n, H, dv)
+        og = r[:, 2 * H * dk + H * dv:]
+        pre = gates.float() + b_gates.float()
+        squashed = cap * torch.tanh(pre / cap)
+        log_in, log_keep = squashed[:, :H], torch.nn.functional.logsigmoid(squashed[:, H:])
+        out = torch.empty(n, H, dv, dtype=torch.float32, device=rows.device)
+        cu = ctx.cu_seqlens.tolist()
+        slots, phase = ctx.state_slots.tolist(), ctx.state_phase.tolist()
+        for s in range(len(cu) - 1):
+            st = state[slots[s], phase[s]].float()
+            C = st[:, : dk * dv].reshape(H, dk, dv).clone()
+            nn_ = st[:, dk * dv: dk * dv + dk].clone()
+            m = st[:, dk * dv + dk].clone()
+            for t in range(cu[s], cu[s + 1]):
+                m_new = torch.maximum(log_keep[t] + m, log_in[t])
+                keep, take = torch.exp(log_keep[t] + m - m_new), torch.exp(log_in[t] - m_new)
+                C = keep[:, None, None] * C + take[:, None, None] * (k[t][:, :, None] * v[t][:, None, :])
+                nn_ = keep[:, None] * nn_ + take[:, None] * k[t]
+                m = m_new
+                den = torch.maximum((nn_ * q[t]).sum(-1).abs(), torch.exp(-m)) + floor
+                out[t] = torch.einsum("hkv,hk->hv", C, q[t]) / den[:, None]
+            state[slots[s], 1 - phase[s]] = torch.cat([C.reshape(H, dk * dv), nn_, m[:, None]], dim=1).to(state.dtype)
+        o = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps)
+        o = o.reshape(n, H * dv) * norm_weight.float() * torch.sigmoid(og)
+        return o.to(rows.dtype)
+
     # ------------------------------------------------------------------ norms
     def materialize(self, delta):
         """The tensor a branch output that is not formed yet stands for (float32)."""
@@ -367,6 +438,34 @@ class ReferenceOps:
             values_t(kv_cache)[page, :, :, off] = v.to(kv_cache.dtype)
         return q.to(dt)
 
+    def qkv_span_prepare(self, rows, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, page_dim: int,
+                         own_kv: bool, prep, positions, kv_cache, slot_mapping):
+        """``rows``: ``[N, Hq dk]`` (queries only) or, with ``own_kv``, ``[N, Hq dk + Hk dk + Hk dv]``.  One RMS norm
+        over all of a token's queries and one over all its keys (``prep.norm_weight_q`` / ``_k`` of those sizes,
+        ``prep.norm_eps``), the queries times ``prep.query_scale``'s position-dependent factor; keys and values
+        written into their pages (if ``kv_cache`` is given) with heads of ``page_dim`` elements, zeros behind the real
+        ones.  Returns q ``[N, Hq, page_dim]`` in the run dtype."""
+        n = rows.shape[0]
+        dt = rows.dtype
+        hq, hk, dk, dv, D = num_heads, num_kv_heads, head_dim, value_dim, page_dim
+        r = rows.float()
+        rms = lambda x, w: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + prep.norm_eps) * w.float()
+        q = rms(r[:, : hq * dk], prep.norm_weight_q)
+        if prep.query_scale is not None:
+            floor_scale, attn_scale = prep.query_scale
+            q = q * (1.0 + attn_scale * torch.log1p(torch.floor((positions.float() + 1.0) / floor_scale)))[:, None]
+        pad = lambda t: torch.nn.functional.pad(t, (0, D - t.shape[-1]))
+        if kv_cache is not None:
+            if not own_kv:
+                raise ValueError("rows without keys and values cannot fill pages")
+            k = rms(r[:, hq * dk: (hq + hk) * dk], prep.norm_weight_k).reshape(n, hk, dk)
+            v = r[:, (hq + hk) * dk:].reshape(n, hk, dv)
+            ps = kv_cache.shape[3]
+            page, off = (slot_mapping // ps).long(), (slot_mapping % ps).long()
+            kv_cache[page, 0, :, off] = pad(k).to(kv_cache.dtype)
+            values_t(kv_cache)[page, :, :, off] = pad(v).to(kv_cache.dtype)
+        return pad(q.reshape(n, hq, dk)).to(dt).contiguous()
+
     def attention_from_qkv(self, qkv, num_heads, num_kv_heads, head_dim, positions, token_segment, prep, kv_cache,
                            writes: bool, slot_mapping, block_table, retention, scale: float, meta=None):
         """q and k prepared, k and v written (if this run writes its cache), attention over the pages."""
@@ -374,9 +473,12 @@ class ReferenceOps:
                                      kv_cache if writes else None, slot_mapping)
         return self.paged_attention(q, kv_cache, block_table, positions, token_segment, retention, scale, meta)
 
-    def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
+    def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None,
+                        bias=None, sink=None):
         """For each token: softmax over the keys of its own request at positions
-        ``[start(pos), pos]``, read from the pages its block table names."""
+        ``[start(pos), pos]``, read from the pages its block table names.  ``bias``: float32 ``[Hq, L]``; a key ``n``
+        places back adds ``bias[h, min(n, L - 1)]`` to head ``h``'s scaled score.  ``sink``: float32 ``[Hq]``;
+        ``exp(sink[h])`` is one more term of head ``h``'s denominator (no key, no value, not scaled, no bias)."""
         n, hq, dh = q.shape
         hk, ps = kv_cache.shape[2], kv_cache.shape[3]
         g = hq // hk
@@ -394,7 +496,16 @@ class ReferenceOps:
             v = values_t(kv_cache)[pages, :, :, off].float()
             qi = q[i].float().reshape(hk, g, dh)
             sc = torch.einsum("hgd,thd->hgt", qi, k) * scale
-            pr = torch.softmax(sc, dim=-1)
+            if bias is not None:
+                back = (p - kpos).clamp_max(bias.shape[1] - 1)
+                sc = sc + bias.float()[:, back].reshape(hk, g, -1)
+            if sink is None:
+                pr = torch.softmax(sc, dim=-1)
+            else:
+                sk = sink.float().reshape(hk, g, 1)
+                top = torch.maximum(sc.max(dim=-1, keepdim=True).values, sk)
+                e = torch.exp(sc - top)
+                pr = e / (e.sum(dim=-1, keepdim=True) + torch.exp(sk - top))
             out[i] = torch.einsum("hgt,thd->hgd", pr, v).reshape(-1).to(q.dtype)
         return out
 
@@ -411,9 +522,10 @@ class ReferenceOps:
         return (ids, gates, None) if group else (ids, gates)
 
     def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None,
-                    shared_weights=None):
+                    shared_weights=None, shared_gate=None):
         """``sum_j  W_down[e_j] (silu(g_j W_gate[e_j] h) * (g_j W_up[e_j] h))`` per token,
-        plus ``shared`` if given; float32 result.  ``w_gate_up`` is ``[E, 2F, D]`` (gate rows then
+        plus ``shared`` if given (``shared_gate = (h32, w)``: times ``sigmoid(h32 . w)``, one float32 number a
+        token); float32 result.  ``w_gate_up`` is ``[E, 2F, D]`` (gate rows then
         up rows), ``w_down`` ``[E, D, F]``.  Activations between the two products are
         rounded to the run dtype, as the kernels store them."""
         assert not tiled, "the plain ops read row-major weights"
@@ -430,6 +542,9 @@ class ReferenceOps:
                 act = (torch.nn.functional.silu(gu[:, :f]) * gu[:, f:]).to(h.dtype).float()
                 out[rows] += (act @ w_down[e].float().t()).to(h.dtype).float()
         if shared is not None:
+            if shared_gate is not None:
+                h32, w = shared_gate
+                shared = (shared.float() * torch.sigmoid(h32.float() @ w.float().reshape(-1, 1))).to(shared.dtype)
             out += shared.float()
         return out
 

@@ -10,16 +10,37 @@ v, directly behind the projection: ``y[t] = sum_j w[:, j] * u[t - taps + 1 + j]`
 start; the last ``taps - 1`` projected rows of every request are its state, kept in two halves so that a step that
 is run twice reads what the first run read) and ``value_dim`` (values of another size than queries and keys: the
 pages then hold heads of the larger of the two sizes, rounded up to a multiple of 8, filled up with zeros, and
-the output projection skips the zeros).  Formulas:
+the output projection skips the zeros).  A second family of options, off for Llama 4 as well: a q/k norm whose
+``span`` is ``"projection"`` (one RMS norm over all heads' queries at once, and one over all keys, weights of that
+size), ``distance_bias`` (a learned number per head and distance added to the scaled score;
+``log_buckets``: a table of ``rows`` rows, the first half one distance each, the other half spread evenly over the
+logarithm of the distance up to ``max_distance``, where the last row begins), ``sink`` (a learned number per head
+whose exponential is one more term of the softmax's denominator) and ``own_kv = False`` (the layer projects no keys
+and values: its run reads the cache that another run writes).  With any of these the rows go through
+``qkv_span_prepare`` (norms over the projections, query scale, pages with heads filled up with zeros) and the
+attention kernels that take a bias table and sinks.  Formulas:
 ``llama4/llama4_jax/model.py:891-955`` (projections, rotation, q/k norm, order of
 the cache write) and ``model.py:745-794`` (scores times ``softmax_scale``, causal
 mask, float32 softmax, values).
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from .base import CacheNeed, Mixer, ParamSpec, QKPreparation, build_position, first_needed_position, register_mixer
+
+
+def log_bucket(distance: int, rows: int, max_distance: int) -> int:
+    """The row of a distance table of ``rows`` rows for a key ``distance`` places back: below ``rows // 2`` every
+    distance has its row; from there the rows are spread evenly over ``ln(distance)`` so that the last one begins at
+    ``max_distance`` (float64)."""
+    half = rows // 2
+    if distance < half:
+        return distance
+    return min(rows - 1, half + int(math.floor(math.log(distance / half) / math.log(max_distance / half)
+                                               * (rows - half))))
 
 
 @register_mixer("attention")
@@ -41,6 +62,20 @@ class Attention(Mixer):
         self.qk_norm_eps = None if qk_norm is None else float(qk_norm.eps)
         self.qk_norm_weighted = bool(qk_norm is not None and qk_norm.get("weighted", False))
         self.qk_norm_first = bool(qk_norm is not None and qk_norm.get("before_rotation", False))
+        self.qk_norm_span = "head" if qk_norm is None else str(qk_norm.get("span") or "head")
+        if self.qk_norm_span not in ("head", "projection"):
+            raise ValueError(f"a q/k norm spans a head or the projection, not {self.qk_norm_span!r}")
+        db = spec.get("distance_bias")
+        if db is not None and db.kind != "log_buckets":
+            raise ValueError(f"unknown distance_bias kind {db.kind!r}")
+        self.bias_rows = None if db is None else int(db.rows)
+        self.bias_max = None if db is None else int(db.max_distance)
+        if db is not None and not 2 <= self.bias_rows // 2 < self.bias_max:
+            raise ValueError("a log_buckets distance table needs at least 4 rows and a max_distance beyond half of them")
+        self.has_sink = bool(spec.get("sink", False))
+        self.own_kv = bool(spec.get("own_kv", True))
+        # the path through the kernel that norms over whole projections, and the attention kernels with bias and sink
+        self.spanned = (self.qk_norm_span == "projection" or db is not None or self.has_sink or not self.own_kv)
         qs = spec.get("query_scale")
         if qs is not None and qs.kind != "log_floor_temperature":
             raise ValueError(f"unknown query_scale kind {qs.kind!r}")
@@ -50,22 +85,40 @@ class Attention(Mixer):
         self.value_dim = int(spec.get("value_dim") or self.head_dim)
         self.biased = bool(spec.get("bias", False))
         self.conv_taps = int(spec.get("conv_taps") or 0)
-        # the path through the convolution kernel, which also rotates, norms, fills up and writes the pages
         rot = self.position.rotation()
-        self.convolved = (self.conv_taps > 0 or self.value_dim != self.head_dim or self.biased
-                          or (rot is not None and rot.magnitude != 1.0))
+        if self.spanned:
+            if self.qk_norm_span != "projection" or not self.qk_norm_weighted or self.qk_norm_first:
+                raise ValueError("distance_bias, sink and own_kv=False come with a weighted q/k norm over the projection")
+            if rot is not None or self.biased or self.conv_taps:
+                raise ValueError("the attention mixer's path with a q/k norm over the projection has no rotation, no "
+                                 "projection bias and no convolution")
+        # the path through the convolution kernel, which also rotates, norms, fills up and writes the pages
+        self.convolved = not self.spanned and (self.conv_taps > 0 or self.value_dim != self.head_dim or self.biased
+                                               or (rot is not None and rot.magnitude != 1.0))
         if self.convolved and (self.qk_norm_weighted or self.qk_norm_first or self.query_scale is not None):
             raise ValueError("the attention mixer's convolution path norms q and k without weights after the rotation "
                              "and has no query scale")
         # the head size of the pages
         self.page_dim = self.head_dim if not self.convolved else -(-max(self.head_dim, self.value_dim) // 8) * 8
+        if self.spanned:  # (from 32 on a multiple of 32: the sizes the matrix-core attention kernels take)
+            widest = max(self.head_dim, self.value_dim)
+            self.page_dim = -(-widest // 32) * 32 if widest >= 32 else -(-widest // 8) * 8
         self.state_dtype = None
+        self.bias_table = None
 
     def param_specs(self):
         hq, hk, dh, d = self.num_heads, self.num_kv_heads, self.head_dim, self.hidden
         dv = self.value_dim
-        channels = (hq + hk) * dh + hk * dv
+        channels = self.channels
         extra = {}
+        if self.spanned:
+            extra["q_norm"] = ParamSpec((hq * dh,), policy="float32", init=("uniform", 0.5, 1.5))
+            if self.own_kv:
+                extra["k_norm"] = ParamSpec((hk * dh,), policy="float32", init=("uniform", 0.5, 1.5))
+            if self.bias_rows is not None:
+                extra["rel"] = ParamSpec((self.bias_rows, hq), policy="float32", init=("normal", 1.0))
+            if self.has_sink:
+                extra["sink"] = ParamSpec((hq,), policy="float32", init=("normal", 1.0))
         if self.biased:
             extra["bqkv"] = ParamSpec((channels,), policy="float32", init=("normal", 0.3))
         if self.conv_taps:
@@ -76,12 +129,22 @@ class Attention(Mixer):
             "wo": ParamSpec((d, hq * dv)),
             **extra,
             **({"q_norm": ParamSpec((dh,), policy="float32", init=("ones",)),
-                "k_norm": ParamSpec((dh,), policy="float32", init=("ones",))} if self.qk_norm_weighted else {}),
+                "k_norm": ParamSpec((dh,), policy="float32", init=("ones",))}
+               if self.qk_norm_weighted and not self.spanned else {}),
         }
 
     @property
     def channels(self) -> int:
+        if not self.own_kv:  # (queries only)
+            return self.num_heads * self.head_dim
         return (self.num_heads + self.num_kv_heads) * self.head_dim + self.num_kv_heads * self.value_dim
+
+    def distance_table(self) -> torch.Tensor:
+        """The learned table told per head and distance, float32 ``[heads, max_distance + 1]``: column ``n`` is what a
+        key ``n`` places back adds to the score, the last column what every key further back adds."""
+        rel = self.params["rel"]
+        row_of = [log_bucket(n, self.bias_rows, self.bias_max) for n in range(self.bias_max + 1)]
+        return rel[torch.tensor(row_of, device=rel.device)].t().contiguous()
 
     def allocate(self, dtype, device) -> None:
         super().allocate(dtype, device)
@@ -96,12 +159,15 @@ class Attention(Mixer):
     graph_safe = True
 
     def finalize(self) -> None:
+        if self.spanned:
+            self.bias_table = self.distance_table() if self.bias_rows is not None else None
         rot = self.position.rotation()
         if rot is not None:
             rot.inv_freq = rot.inv_freq.to(self.params["wqkv"].device)
         self.prep.rotation = rot
         self.prep.norm_weight_q = self.params.get("q_norm")
         self.prep.norm_weight_k = self.params.get("k_norm")
+        self.prep.norm_span = self.qk_norm_span
         self.bias_run = None
         if self.biased:  # (the library's product adds a bias of its operands' dtype)
             self.bias_run = self.params["bqkv"].to(self.params["wqkv"].dtype)
@@ -121,6 +187,17 @@ class Attention(Mixer):
 
     def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
         ops = ctx.ops
+        if self.spanned:
+            if cache.writes != self.own_kv:
+                raise ValueError("a run writes its cache if and only if its layer projects keys and values")
+            rows = ops.linear(h, self.params["wqkv"])
+            q = ops.qkv_span_prepare(rows, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim,
+                                     self.page_dim, self.own_kv, self.prep, ctx.positions,
+                                     cache.kv if cache.writes else None, cache.slot_mapping)
+            o = ops.paged_attention(q, cache.kv, cache.block_table, ctx.positions, ctx.token_segment, self.retention,
+                                    self.softmax_scale, cache.attn_meta, bias=self.bias_table,
+                                    sink=self.params.get("sink"))
+            return ops.linear(o, self.params["wo"] if self.wo_padded is None else self.wo_padded)
         if self.convolved:
             # the projection (its bias added by the product where the library does it, else by the kernel that reads
             # the rows next); then convolution from the rows and the request's state, rotation, norm, pages, attention

@@ -253,6 +253,7 @@ class QKPreparation:
     norm_weight_k: Optional[torch.Tensor] = None
     norm_first: bool = False  # the norm comes before the rotation
     query_scale: Optional[tuple] = None  # (floor_scale, attn_scale): q *= 1 + attn_scale * ln(1 + floor((pos + 1) / floor_scale))
+    norm_span: str = "head"  # "projection": one norm over all heads' queries, one over all keys (weights of that size)
 
     @property
     def plain(self) -> bool:
@@ -260,7 +261,8 @@ class QKPreparation:
         r = self.rotation
         return ((r is None or (r.pairing == "adjacent" and r.rotary_dim in (0, 2 * r.inv_freq.numel())
                                and r.magnitude == 1.0))
-                and self.norm_weight_q is None and self.norm_weight_k is None and not self.norm_first)
+                and self.norm_weight_q is None and self.norm_weight_k is None and not self.norm_first
+                and self.norm_span == "head")
 
 
 class PositionEncoding:

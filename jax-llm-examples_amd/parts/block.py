@@ -38,22 +38,25 @@ class PreNormBlock:
     def __init__(self, spec: LayerSpec) -> None:
         self.spec = spec
         self.mixer = build_mixer(spec.mixer)
-        self.feed_forward = build_feed_forward(spec.feed_forward)
         self.mixer_norm = build_norm(spec.mixer_norm)
-        self.feed_forward_norm = build_norm(spec.feed_forward_norm)
+        self.feed_forward = self.feed_forward_norm = None  # (a layer may have no feed-forward)
+        if spec.feed_forward is not None:
+            self.feed_forward = build_feed_forward(spec.feed_forward)
+            self.feed_forward_norm = build_norm(spec.feed_forward_norm)
 
     def parts(self):
-        return {
-            "mixer": self.mixer,
-            "feed_forward": self.feed_forward,
-            "mixer_norm": self.mixer_norm,
-            "feed_forward_norm": self.feed_forward_norm,
-        }
+        out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm}
+        if self.feed_forward is not None:
+            out.update(feed_forward=self.feed_forward, feed_forward_norm=self.feed_forward_norm)
+        return out
 
     def forward(self, residual, ctx, cache) -> None:
-        h, _ = self.mixer_norm.forward(residual, ctx)
-        residual.add(self.mixer.forward(h, ctx, cache))
+        want32 = bool(getattr(self.mixer, "wants_float32_input", False))
+        h, h32 = self.mixer_norm.forward(residual, ctx, want32=want32)
+        residual.add(self.mixer.forward(h, ctx, cache, h32) if want32 else self.mixer.forward(h, ctx, cache))
         ff = self.feed_forward
+        if ff is None:
+            return
         if getattr(ff, "accepts_deferred_norm", False):  # (it hands the rows to the kernel set only: see there)
             h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=ff.wants_float32_input, defer=True)
         else:
@@ -200,3 +203,68 @@ class SandwichGatedBlock:
         post = self.feed_forward_post_norm
         residual.add(GatedBranch(y, bias, gate, self.feed_forward_gate.params["bias"], post.params.get("weight"),
                                  post.eps))
+
+
+class StreamWeights(Part):
+    """What one branch of a layer over several residual streams learns about them: ``inw`` (how the branch's input
+    is put together from the streams), ``mix`` (``[from, to]``: how the streams are mixed among themselves when the
+    branch's output arrives) and ``outw`` (how much of the output every stream takes).  All float32."""
+
+    graph_safe = True
+
+    def __init__(self, streams: int) -> None:
+        super().__init__()
+        self.streams = int(streams)
+
+    def param_specs(self):
+        s = self.streams
+        return {"inw": ParamSpec((s,), policy="float32", init=("uniform", 0.2, 0.8)),
+                "outw": ParamSpec((s,), policy="float32", init=("uniform", 0.3, 1.0)),
+                "mix": ParamSpec((s, s), policy="float32", init=("uniform", 0.0, 2.0 / s))}
+
+    def flops_per_token(self) -> float:
+        return 0.0
+
+
+@register_arrangement("hyper_streams")
+class HyperStreamsBlock:
+    """Pre-norm branches over ``S`` residual streams (the plan's residual kind ``streams``)::
+
+        u = sum_s inw[s] X_s;   y = branch(norm(u));   X_t <- sum_s mix[s, t] X_s + outw[t] y
+
+    for the mixer and then for the feed-forward, each with stream weights of its own (``hc1``, ``hc2``).  The update
+    stays pending on the streams; the kernel that forms the next branch's input makes it first.  The layer may have
+    no feed-forward.  Options (``LayerSpec.options``): ``streams``."""
+
+    def __init__(self, spec: LayerSpec) -> None:
+        self.spec = spec
+        s = int(spec.options["streams"])
+        self.mixer = build_mixer(spec.mixer)
+        self.mixer_norm = build_norm(spec.mixer_norm)
+        self.hc1 = StreamWeights(s)
+        self.feed_forward = self.feed_forward_norm = self.hc2 = None
+        if spec.feed_forward is not None:
+            self.feed_forward = build_feed_forward(spec.feed_forward)
+            self.feed_forward_norm = build_norm(spec.feed_forward_norm)
+            self.hc2 = StreamWeights(s)
+
+    def parts(self):
+        out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm, "hc1": self.hc1}
+        if self.feed_forward is not None:
+            out.update(feed_forward=self.feed_forward, feed_forward_norm=self.feed_forward_norm, hc2=self.hc2)
+        return out
+
+    def forward(self, residual, ctx, cache) -> None:
+        if not hasattr(residual, "branch_input"):
+            raise TypeError("the hyper_streams arrangement works on the residual kind 'streams'")
+        hc, norm = self.hc1.params, self.mixer_norm
+        want32 = bool(getattr(self.mixer, "wants_float32_input", False))
+        h, h32 = residual.branch_input(ctx, hc["inw"], norm.params.get("weight"), norm.eps, want32)
+        y = self.mixer.forward(h, ctx, cache, h32) if want32 else self.mixer.forward(h, ctx, cache)
+        residual.add_update(y, hc["mix"], hc["outw"])
+        ff = self.feed_forward
+        if ff is None:
+            return
+        hc, norm = self.hc2.params, self.feed_forward_norm
+        h, h32 = residual.branch_input(ctx, hc["inw"], norm.params.get("weight"), norm.eps, ff.wants_float32_input)
+        residual.add_update(ff.forward(h, h32, ctx), hc["mix"], hc["outw"])

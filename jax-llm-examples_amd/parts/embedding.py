@@ -1,7 +1,9 @@
 """The two ends of a decoder: token embedding and output head.
 
 ``token_embedding`` (``llama4/llama4_jax/model.py:1195``): row ``token`` of the table, as the first
-value of the float32 residual; optionally times a constant (``multiplier``).
+value of the float32 residual; optionally times a constant (``multiplier``), and optionally plus a sinusoidal
+position vector (``sinusoid`` = its base ``b``): entry ``2i`` is ``sin(pos * b^(-2i/hidden))``, entry ``2i + 1`` the
+cosine of the same angle (the rates formed once in float64 and rounded, the angles float32).
 ``token_pair_embedding``: the token's row plus a row of a second table chosen by a hash of (token before, token):
 ``(prev * mul_prev + token * mul_cur) mod buckets``, and the table's extra last row for a sequence's first token.
 The token before is known to the step (``StepContext.prev_token_ids``; across steps the cache manager keeps it).
@@ -23,6 +25,9 @@ class TokenEmbedding(Embedding):
         self.vocab_size, self.hidden = int(spec.vocab_size), int(spec.hidden_size)
         m = spec.get("multiplier")
         self.multiplier = None if m is None else float(m)
+        b = spec.get("sinusoid")
+        self.sinusoid_base = None if b is None else float(b)
+        self.rates = None
 
     graph_safe = True
 
@@ -32,7 +37,16 @@ class TokenEmbedding(Embedding):
     def flops_per_token(self) -> float:
         return 0.0
 
+    def finalize(self) -> None:
+        if self.sinusoid_base is not None and self.rates is None:
+            i = torch.arange((self.hidden + 1) // 2, dtype=torch.float64)
+            rates = torch.tensor(self.sinusoid_base, dtype=torch.float64) ** (-2.0 * i / self.hidden)
+            self.rates = rates.to(torch.float32).to(self.params["weight"].device)
+
     def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+        if self.sinusoid_base is not None:
+            return ctx.ops.embed_sinusoid(token_ids, ctx.positions, self.params["weight"],
+                                          1.0 if self.multiplier is None else self.multiplier, self.rates)
         x = ctx.ops.embed(token_ids, self.params["weight"])
         if self.multiplier is not None:
             x.mul_(self.multiplier)

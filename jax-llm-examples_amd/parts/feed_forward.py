@@ -5,7 +5,8 @@
 gate = sigmoid of the chosen logit, the gate multiplies the expert's *input*
 (``model.py:958-972, 1066-1071``), SwiGLU experts (``model.py:1076-1085``), sum
 over the chosen experts (``model.py:1111``), plus one shared SwiGLU expert on the
-unscaled input (``model.py:1137-1139``).
+unscaled input (``model.py:1137-1139``).  With the option ``shared_gate`` (off for Llama 4) the shared expert's output
+is multiplied by ``sigmoid(w_sg . h)``, one number a token, formed in float32.
 """
 from __future__ import annotations
 
@@ -56,6 +57,9 @@ class MoESigmoidShared(FeedForward):
         self.top_k = int(spec.top_k)
         self.inter = int(spec.intermediate_size)
         self.shared_inter = int(spec.get("shared_intermediate_size") or 0)
+        self.shared_gate = bool(spec.get("shared_gate", False))
+        if self.shared_gate and not self.shared_inter:
+            raise ValueError("a shared expert's gate needs a shared expert")
         self.tiled = False  # expert matrices are in the kernels' streaming layout (ops/layout.py)
 
     def param_specs(self):
@@ -68,6 +72,8 @@ class MoESigmoidShared(FeedForward):
         if self.shared_inter:
             specs["shared_gate_up"] = ParamSpec((2 * self.shared_inter, d))
             specs["shared_down"] = ParamSpec((d, self.shared_inter))
+        if self.shared_gate:
+            specs["shared_gate"] = ParamSpec((1, d), policy="float32")
         return specs
 
     graph_safe = True
@@ -107,6 +113,10 @@ class MoESigmoidShared(FeedForward):
                 expert_ids, gates = replaced
                 grouping = None
         shared = (self.params["shared_gate_up"], self.params["shared_down"]) if self.shared_inter else None
+        if self.shared_gate:
+            return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"],
+                                   shared_weights=shared, tiled=self.tiled, grouping=grouping,
+                                   shared_gate=(h32, self.params["shared_gate"]))
         return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"],
                                shared_weights=shared, tiled=self.tiled, grouping=grouping)
 

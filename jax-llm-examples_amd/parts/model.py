@@ -7,7 +7,7 @@ import torch
 
 from ..cache.manager import CacheView
 from ..config.specs import ModelPlan
-from .residual import Residual
+from .residual import build_residual
 from ..config.specs import part
 from . import embedding as _ends  # noqa: F401  (registers the built-in embedding and head)
 from .base import CacheNeed, ParamSpec, Part, build_embedding, build_head, build_norm
@@ -94,7 +94,7 @@ class DecoderModel:
         """Runs the step's tokens through every run of the order; returns float32
         logits ``[len(ctx.logits_indices), vocab]``."""
         ops = ctx.ops
-        residual = Residual(self.embed.forward(ctx.token_ids, ctx))
+        residual = build_residual(self.plan.residual, self.embed.forward(ctx.token_ids, ctx))
         embedded = None
         if self.loop is not None and getattr(self.loop, "needs_embedding_output", False):
             embedded = residual.x.clone()  # (the stream itself is added to in place)

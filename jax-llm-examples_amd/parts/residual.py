@@ -1,6 +1,12 @@
 """The residual stream of a step: float32 rows plus at most one pending branch
 output.  The sum is applied by the next norm (one kernel does add and norm) or
-when the value is asked for."""
+when the value is asked for.
+
+A plan may name another kind of stream (``ModelPlan.residual``).  ``streams``: ``S`` copies ``X_1 .. X_S`` of the
+stream, all equal to the embedding's output at the start; a branch reads ``u = sum_s a_s X_s`` through its norm, and
+its output ``y`` changes all copies at once, ``X_t <- sum_s M[s, t] X_s + o_t y``; at the model's end the copies are
+added up.  ``a``, ``M`` and ``o`` belong to the branch (:class:`~.block.StreamWeights`).  The update stays pending
+until the kernel that forms the next branch's input makes it."""
 from __future__ import annotations
 
 import torch
@@ -117,3 +123,79 @@ class Residual:
             else:
                 r.pending = ctx.ops.gather_rows(self.pending, idx)
         return r
+
+
+class StreamUpdate:
+    """A branch output ``y`` that is still to be worked into the streams: ``X_t <- sum_s mix[s, t] X_s + outw[t] y``."""
+
+    def __init__(self, y, mix, outw) -> None:
+        self.y, self.mix, self.outw = y, mix, outw
+
+
+class StreamsResidual:
+    """``S`` residual streams, float32 ``[N, S, hidden]``.  What the other kind offers where the model and the norms
+    use it (``value``, ``rows``, ``normed``: all about the sum of the streams), and for the arrangement that knows of
+    streams ``branch_input`` / ``add_update``."""
+
+    def __init__(self, xs: torch.Tensor) -> None:
+        assert xs.dtype == torch.float32 and xs.dim() == 3
+        self.xs = xs
+        self.streams = xs.shape[1]
+        self.pending = None
+
+    @classmethod
+    def start(cls, x: torch.Tensor, streams: int) -> "StreamsResidual":
+        """Every stream a copy of the embedding's output."""
+        return cls(x.unsqueeze(1).expand(-1, int(streams), -1).contiguous())
+
+    def add_update(self, y, mix, outw) -> None:
+        if self.pending is not None:
+            raise AssertionError("a branch output is already pending on the streams")
+        if tuple(y.shape) != (self.xs.shape[0], self.xs.shape[2]):
+            raise ValueError(f"branch output {tuple(y.shape)} does not match streams {tuple(self.xs.shape)}")
+        self.pending = StreamUpdate(y, mix, outw)
+
+    def branch_input(self, ctx, inw, weight, eps: float, want32: bool = False):
+        """Makes the pending update, then ``u = sum_s inw[s] X_s`` (``inw`` ``None``: the plain sum) and its RMS
+        norm with ``weight``; one kernel.  Returns ``(h, h in float32 or None)``."""
+        h, h32 = ctx.ops.streams_mix_norm(self.xs, self.pending, inw, weight, eps, ctx.dtype, want32)
+        self.pending = None
+        return h, h32
+
+    def normed(self, ctx, weight, eps: float, want32: bool = False, defer: bool = False):
+        """The norm of the streams' sum (what the model's final norm asks for)."""
+        return self.branch_input(ctx, None, weight, eps, want32)
+
+    def value(self, ctx) -> torch.Tensor:
+        """The sum of the streams, with what is pending worked in."""
+        if self.pending is not None:
+            ctx.ops.streams_mix_norm(self.xs, self.pending, None, None, 0.0, ctx.dtype, False, norm=False)
+            self.pending = None
+        return self.xs.sum(dim=1)
+
+    @property
+    def x(self) -> torch.Tensor:
+        return self.xs.sum(dim=1)
+
+    def rows(self, ctx, idx: torch.Tensor) -> "StreamsResidual":
+        """The streams of the chosen rows only (what is pending stays pending)."""
+        n, s, d = self.xs.shape
+        r = StreamsResidual(ctx.ops.gather_rows(self.xs.view(n, s * d), idx).view(-1, s, d))
+        if self.pending is not None:
+            p = self.pending
+            r.pending = StreamUpdate(ctx.ops.gather_rows(p.y, idx), p.mix, p.outw)
+        return r
+
+
+_RESIDUALS = {"streams": lambda spec, x: StreamsResidual.start(x, spec.streams)}
+
+
+def build_residual(spec, x: torch.Tensor):
+    """The residual stream of a step from the embedding's output ``x`` (float32 ``[N, hidden]``), of the kind the plan
+    names (``None``: the plain one)."""
+    if spec is None:
+        return Residual(x)
+    try:
+        return _RESIDUALS[spec.kind](spec, x)
+    except KeyError:
+        raise KeyError(f"unknown residual kind {spec.kind!r}; known: {sorted(_RESIDUALS)}") from None

@@ -14,7 +14,8 @@ class TensorBinding:
     (a key of ``DecoderModel.named_parameters()``).  ``transpose``: two axes of
     the stored tensor to swap first.  ``rows``: the range of the target's first
     axis it fills (the whole target if ``None``) - several tensors can fill one
-    fused parameter.  ``init``: how seeded random weights draw it.
+    fused parameter.  ``index``: which slice of the target's leading axis is meant
+    before ``rows`` applies (one expert's matrix of a stacked parameter).  ``init``: how seeded random weights draw it.
     """
 
     name: str
@@ -23,4 +24,5 @@ class TensorBinding:
     transpose: Optional[tuple[int, int]] = None
     rows: Optional[tuple[int, int]] = None
     init: tuple = ("normal", 0.02)
+    index: Optional[int] = None
     float32: bool = False  # stored in 32-bit by the random-weights writer whatever the run dtype

@@ -55,6 +55,19 @@ def _checkpoint_files(model_dir: str) -> list[str]:
     return files
 
 
+def checkpoint_shapes(model_dir: str, optional_prefixes: Sequence[str] = ()) -> dict:
+    """The stored shape of every tensor of a model folder, by name (the files' headers only are read)."""
+    out = {}
+    for path in _checkpoint_files(os.fspath(model_dir)):
+        f = SafetensorsFile(path)
+        try:
+            for raw in f.names():
+                out.setdefault(_canonical(raw, optional_prefixes), tuple(f.shape(raw)))
+        finally:
+            f.close()
+    return out
+
+
 def _canonical(name: str, optional_prefixes: Sequence[str]) -> str:
     for p in optional_prefixes:
         if name.startswith(p):
@@ -111,6 +124,8 @@ def place(target: torch.Tensor, b: TensorBinding, t: torch.Tensor) -> None:
         t = t.to(torch.int32)
     if b.transpose is not None:
         t = t.transpose(*b.transpose)
+    if b.index is not None:
+        target = target[b.index]
     dst = target if b.rows is None else target[b.rows[0]: b.rows[1]]
     if tuple(dst.shape) != tuple(t.shape):
         raise AssertionError(f"binding {b.name}: {tuple(t.shape)} does not fit {b.target}{tuple(dst.shape)}")
