@@ -44,7 +44,8 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ kv, T* __restrict__ out, const int* __restrict__ positions,
     const int* __restrict__ token_segment, const int* __restrict__ block_table, int table_width, int ret_mode,
     int ret_param, float scale, int N, int Hq, int Hkv, int dh, int ps, int splits, int tiles_per_split,
-    float* __restrict__ ws_ml, float* __restrict__ ws_o) {
+    float* __restrict__ ws_ml, float* __restrict__ ws_o, const float* __restrict__ bias, int bias_len,
+    const float* __restrict__ sink) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave_index();
   if (item >= N * Hq * splits) return;  // whole wavefront leaves; no block-wide barrier below
@@ -92,6 +93,8 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
           for (int i = 0; i < Vec16<T>::kN; ++i) dot += qv.get(i) * kvv.get(i);
         }
         s = dot * scale;
+        // a learned number per head and distance; every key further back than the table is long takes its last entry
+        if (bias != nullptr) s += bias[(size_t)h * bias_len + min(pos - key, bias_len - 1)];
       }
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -166,6 +169,8 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     }
     return;
   }
+  // the sink: one more term of the denominator, without a key or a value
+  if (sink != nullptr) l += expf(sink[h] - m);
   const float inv = bad ? __builtin_nanf("") : 1.0f / l;
   T* o = out + ((size_t)n * Hq + h) * dh;
 #pragma unroll
@@ -180,7 +185,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void paged_attention_generic_merge_kernel(const float* __restrict__ ws_ml,
                                                                             const float* __restrict__ ws_o,
                                                                             T* __restrict__ out, int NH, int dh,
-                                                                            int splits) {
+                                                                            int splits, const float* __restrict__ sink,
+                                                                            int Hq) {
   const int lane = threadIdx.x & 63;
   const int nh = blockIdx.x * 4 + wave_index();
   if (nh >= NH) return;
@@ -224,6 +230,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_merge_kernel(cons
       for (int i = 0; i < 4; ++i) acc[i] += o[u][i] * wgt;
     }
   }
+  if (sink != nullptr) l += expf(sink[nh % Hq] - mx);
   const float inv = bad ? __builtin_nanf("") : 1.0f / l;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -235,12 +242,15 @@ __global__ __launch_bounds__(256) void paged_attention_generic_merge_kernel(cons
 // splits > 1 (few tokens with many keys: decode): every (token, head) is shared between `splits` wavefronts,
 // tiles_per_split tiles of 64 keys each, and merged by a second kernel; ws_ml: [N * Hq * splits * 2] float32,
 // ws_o: [N * Hq * splits * dh] float32.  splits * tiles_per_split must cover the longest range of keys.
-JLE_API int jle_paged_attention_generic(const void* q, const void* kv, void* out, const int* positions,
-                                        const int* token_segment, const int* block_table, int table_width,
-                                        int ret_mode, int ret_param, float scale, int is_bf16, int N, int Hq, int Hkv,
-                                        int dh, int ps, int splits, int tiles_per_split, float* ws_ml, float* ws_o,
-                                        hipStream_t s) {
+// bias: float32 [Hq][bias_len] or null: a key n places back adds bias[h][min(n, bias_len - 1)] to head h's scaled
+// score; sink: float32 [Hq] or null: exp(sink[h]) is one more term of head h's denominator.
+static int launch_generic(const void* q, const void* kv, void* out, const int* positions, const int* token_segment,
+                          const int* block_table, int table_width, int ret_mode, int ret_param, float scale,
+                          int is_bf16, int N, int Hq, int Hkv, int dh, int ps, int splits, int tiles_per_split,
+                          float* ws_ml, float* ws_o, const float* bias, int bias_len, const float* sink,
+                          hipStream_t s) {
   if (N <= 0) return 0;
+  if (bias != nullptr && bias_len < 1) return JLE_BAD_ARG;
   if (dh % 8 || dh > 256 || Hkv <= 0 || Hq % Hkv || ps <= 0) return JLE_BAD_ARG;
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
   if (splits < 1 || (splits > 1 && (tiles_per_split < 1 || ws_ml == nullptr || ws_o == nullptr))) return JLE_BAD_ARG;
@@ -251,22 +261,40 @@ JLE_API int jle_paged_attention_generic(const void* q, const void* kv, void* out
   if (is_bf16) {
     hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,
                        (bf16_t*)out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale,
-                       N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o);
+                       N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(paged_attention_generic_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * Hq,
-                         dh, splits);
+                         dh, splits, sink, Hq);
   } else {
     hipLaunchKernelGGL(paged_attention_generic_kernel<float>, g, b, 0, s, (const float*)q, (const float*)kv,
                        (float*)out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale, N,
-                       Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o);
+                       Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(paged_attention_generic_merge_kernel<float>, gm, b, 0, s, ws_ml, ws_o, (float*)out, N * Hq, dh,
-                         splits);
+                         splits, sink, Hq);
   }
   JLE_LAUNCH_CHECK();
   return 0;
+}
+
+JLE_API int jle_paged_attention_generic(const void* q, const void* kv, void* out, const int* positions,
+                                        const int* token_segment, const int* block_table, int table_width,
+                                        int ret_mode, int ret_param, float scale, int is_bf16, int N, int Hq, int Hkv,
+                                        int dh, int ps, int splits, int tiles_per_split, float* ws_ml, float* ws_o,
+                                        hipStream_t s) {
+  return launch_generic(q, kv, out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale,
+                        is_bf16, N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, nullptr, 0, nullptr, s);
+}
+
+JLE_API int jle_paged_attention_biased(const void* q, const void* kv, void* out, const int* positions,
+                                       const int* token_segment, const int* block_table, int table_width,
+                                       int ret_mode, int ret_param, float scale, int is_bf16, int N, int Hq, int Hkv,
+                                       int dh, int ps, int splits, int tiles_per_split, float* ws_ml, float* ws_o,
+                                       const float* bias, int bias_len, const float* sink, hipStream_t s) {
+  return launch_generic(q, kv, out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale,
+                        is_bf16, N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink, s);
 }
 
 // The merge alone, for kernels that leave their key ranges' results in the same layout (attention_f32.hip).
@@ -276,9 +304,11 @@ JLE_API int jle_attention_merge(const float* ws_ml, const float* ws_o, void* out
   if (splits < 1 || dh <= 0 || dh > 256 || ws_ml == nullptr || ws_o == nullptr) return JLE_BAD_ARG;
   dim3 gm((unsigned)(((long long)NH + 3) / 4)), b(256);
   if (is_bf16)
-    hipLaunchKernelGGL(paged_attention_generic_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, NH, dh, splits);
+    hipLaunchKernelGGL(paged_attention_generic_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, NH, dh, splits,
+                       nullptr, 1);
   else
-    hipLaunchKernelGGL(paged_attention_generic_merge_kernel<float>, gm, b, 0, s, ws_ml, ws_o, (float*)out, NH, dh, splits);
+    hipLaunchKernelGGL(paged_attention_generic_merge_kernel<float>, gm, b, 0, s, ws_ml, ws_o, (float*)out, NH, dh, splits,
+                       nullptr, 1);
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -78,6 +78,14 @@ _SIGNATURES = {
     "jle_conv_qk_prepare": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _f, _vp, _vp, _i, _i,
                             _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_streams_mix_norm": [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _f, _vp, _i, _vp, _i, _i, _i, _i,
+                             _vp],
+    "jle_embed_sinusoid": [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _vp],
+    "jle_mlstm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _f, _f, _vp],
+    "jle_span_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_row_gate": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
+    "jle_paged_attention_biased": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
+                                   _vp, _vp, _i, _vp, _vp],
 }
 
 
@@ -251,6 +259,82 @@ class HipOps:
         out = torch.empty(n, d, dtype=torch.float32, device=table.device)
         self._call("jle_embed_pair", _p(token_ids), _p(prev_token_ids), _p(table), _p(pair_table), self._is_bf16(table),
                    _p(out), n, d, int(buckets), int(mul_prev), int(mul_cur))
+        return out
+
+    def embed_sinusoid(self, token_ids, positions, table, multiplier: float, rates):
+        """``table[token] * multiplier`` plus the position's sinusoid (entry ``2i``: ``sin(pos * rates[i])``, entry
+        ``2i + 1``: the cosine), float32."""
+        n, (v, d) = token_ids.numel(), table.shape
+        self._chk(token_ids, torch.int32, (n,), "token ids")
+        self._chk(positions, torch.int32, (n,), "positions")
+        self._chk(table, None, (v, d), "embedding table")
+        self._chk(rates, torch.float32, ((d + 1) // 2,), "sinusoid rates")
+        out = torch.empty(n, d, dtype=torch.float32, device=table.device)
+        self._call("jle_embed_sinusoid", _p(token_ids), _p(positions), _p(table), self._is_bf16(table),
+                   float(multiplier), _p(rates), _p(out), n, 1, d)
+        return out
+
+    # ------------------------------------------------------------------ several residual streams
+    MAX_STREAMS = 16
+
+    def streams_mix_norm(self, xs, update, inw, weight, eps: float, out_dtype, want32: bool = False, norm: bool = True):
+        """``xs``: float32 ``[N, S, D]``, changed in place: the pending ``update`` (a branch output, a plain tensor or
+        an :class:`ExpertSum`, with ``mix`` ``[from, to]`` and ``outw``) worked into all streams at once, then the
+        norm of ``sum_s inw[s] X_s`` (``inw`` ``None``: the plain sum); one launch."""
+        n, s_, d = xs.shape
+        self._chk(xs, torch.float32, (n, s_, d), "residual streams")
+        if s_ > self.MAX_STREAMS:
+            raise KernelError(f"the streams kernel takes up to {self.MAX_STREAMS} streams, not {s_}")
+        kind, plain, routed, inv, k, shared, is_bf16, mix, outw = 0, None, None, None, 0, None, 0, None, None
+        if update is not None:
+            y, mix, outw = update.y, update.mix, update.outw
+            self._chk(mix, torch.float32, (s_, s_), "stream mix")
+            self._chk(outw, torch.float32, (s_,), "stream output weights")
+            if isinstance(y, ExpertSum):
+                if tuple(y.shape) != (n, d):
+                    raise KernelError("the branch output does not fit the streams")
+                kind, routed, inv, k, shared = 2, y.routed, y.inv, y.k, y.shared
+                is_bf16 = self._is_bf16(routed)
+            else:
+                self._chk(y, None, (n, d), "branch output")
+                kind, plain, is_bf16 = 1, y, self._is_bf16(y)
+        if inw is not None:
+            self._chk(inw, torch.float32, (s_,), "stream input weights")
+        if weight is not None:
+            self._chk(weight, torch.float32, (d,), "norm weight")
+        out = torch.empty(n, d, dtype=out_dtype, device=xs.device) if norm else None
+        out32 = torch.empty(n, d, dtype=torch.float32, device=xs.device) if norm and want32 else None
+        self._call("jle_streams_mix_norm", _p(xs), kind, _p(plain), _p(routed), _p(inv), k, _p(shared), is_bf16,
+                   _p(mix), _p(outw), _p(inw), _p(weight), float(eps), _p(out),
+                   self._is_bf16(out) if out is not None else 0, _p(out32), n, s_, d, int(bool(norm)))
+        return out, out32
+
+    # ------------------------------------------------------------------ a matrix memory per head
+    def mlstm(self, rows, gates, b_gates, norm_weight, num_heads: int, head_dim: int, value_dim: int, cap: float,
+              eps: float, floor: float, state, ctx):
+        """``rows``: q | k | v | output gate in the run dtype; ``gates``: float32 ``[N, 2 H]`` pre-activations without
+        their biases (overwritten).  Every segment's tokens in order from its request's state (``state[slot, phase]``),
+        the new state to the other half; ``[N, H dv]`` in the run dtype."""
+        n = rows.shape[0]
+        H, dk, dv = num_heads, head_dim, value_dim
+        self._chk(rows, None, (n, 2 * H * dk + 2 * H * dv), "q|k|v|gate rows")
+        self._chk(gates, torch.float32, (n, 2 * H), "gate pre-activations")
+        self._chk(b_gates, torch.float32, (2 * H,), "gate biases")
+        self._chk(norm_weight, torch.float32, (H * dv,), "head norm weight")
+        self._chk(state, torch.float32, (state.shape[0], 2, H, dk * dv + dk + 1), "matrix-memory state")
+        r = ctx.num_segments
+        self._chk(ctx.cu_seqlens, torch.int32, (r + 1,), "segment bounds")
+        self._chk(ctx.state_slots, torch.int32, (r,), "state slots")
+        self._chk(ctx.state_phase, torch.int32, (r,), "state phases")
+        if ctx.num_tokens != n:
+            raise KernelError("the rows do not fit the step")
+        if dv % 4 or dk > 256:
+            raise KernelError(f"matrix-memory kernel: value size {dv} must be a multiple of 4 and key size {dk} at most 256")
+        o_raw = torch.empty(n, H * dv, dtype=torch.float32, device=rows.device)
+        out = torch.empty(n, H * dv, dtype=rows.dtype, device=rows.device)
+        self._call("jle_mlstm", _p(rows), self._is_bf16(rows), _p(gates), _p(b_gates), _p(norm_weight), _p(state),
+                   _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(o_raw), _p(out), n, r, H, dk, dv,
+                   float(cap), float(eps), float(floor))
         return out
 
     def add_norm_pair(self, x, delta, injected, weight_a, weight_b, eps: float, out_dtype, second: bool = False,
@@ -977,6 +1061,35 @@ class HipOps:
                    _p(prep.norm_weight_k), int(bool(prep.norm_first)))
         return q
 
+    def qkv_span_prepare(self, rows, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, page_dim: int,
+                         own_kv: bool, prep, positions, kv_cache, slot_mapping):
+        """One RMS norm over all of a token's queries and one over all its keys (weights of those sizes), the queries
+        times ``prep.query_scale``'s factor, keys and values into their pages with heads of ``page_dim`` elements
+        (zeros behind the real ones).  Returns q ``[N, Hq, page_dim]``."""
+        n = rows.shape[0]
+        hq, hk, dk, dv, pd = num_heads, num_kv_heads, head_dim, value_dim, page_dim
+        width = hq * dk + ((hk * dk + hk * dv) if own_kv else 0)
+        self._chk(rows, None, (n, width), "projected rows")
+        self._chk(positions, torch.int32, (n,), "positions")
+        self._chk(prep.norm_weight_q, torch.float32, (hq * dk,), "q norm weight")
+        if prep.norm_eps is None:
+            raise KernelError("the norm over the projection needs its eps")
+        ps = 1
+        if kv_cache is not None:
+            if not own_kv:
+                raise KernelError("rows without keys and values cannot fill pages")
+            ps = kv_cache.shape[3]
+            self._chk(kv_cache, rows.dtype, (kv_cache.shape[0], 2, hk, ps, pd), "kv pages")
+            self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
+            self._chk(prep.norm_weight_k, torch.float32, (hk * dk,), "k norm weight")
+        q = torch.empty(n, hq, pd, dtype=rows.dtype, device=rows.device)
+        fs, sc = (prep.query_scale if prep.query_scale is not None else (0.0, 0.0))
+        self._call("jle_span_prepare", _p(rows), _p(q), _p(kv_cache), _p(positions),
+                   _p(slot_mapping) if kv_cache is not None else None, _p(prep.norm_weight_q),
+                   _p(prep.norm_weight_k) if kv_cache is not None else None, float(prep.norm_eps), float(fs), float(sc),
+                   self._is_bf16(rows), n, hq, hk, dk, dv, pd, ps, int(bool(own_kv)))
+        return q
+
     TICKETS = 1 << 16
 
     def attention_from_qkv(self, qkv, num_heads, num_kv_heads, head_dim, positions, token_segment, prep, kv_cache,
@@ -1134,7 +1247,10 @@ class HipOps:
     F32_TILE = 16  # tokens per work item of the float32 matrix-instruction attention
     F32_DECODE_ITEMS = 2048  # ... in a step of single tokens: about so many (token, kv head, key range) items
 
-    def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
+    def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None,
+                        bias=None, sink=None):
+        """``bias``: float32 ``[Hq, L]``: a key ``n`` places back adds ``bias[h, min(n, L - 1)]`` to head ``h``'s scaled
+        score; ``sink``: float32 ``[Hq]``: ``exp(sink[h])`` is one more term of head ``h``'s denominator."""
         n, hq, dh = q.shape
         hk, ps = kv_cache.shape[2], kv_cache.shape[3]
         self._chk(q, kv_cache.dtype, None, "q")
@@ -1145,7 +1261,12 @@ class HipOps:
         mode = _ret_mode(retention)
         param = int(retention[1]) if len(retention) > 1 else 0
         out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
-        if (q.dtype == torch.bfloat16 and hq // hk <= 32
+        biased = bias is not None or sink is not None
+        if bias is not None:
+            self._chk(bias, torch.float32, (hq, bias.shape[1]), "distance bias")
+        if sink is not None:
+            self._chk(sink, torch.float32, (hq,), "sinks")
+        if (not biased and q.dtype == torch.bfloat16 and hq // hk <= 32
                 and self._query("jle_attention_mfma_supported", dh, hq, hk, ps)):
             key = f"attn_plan_{hq // hk}"
             plan = meta.meta.get(key) if meta is not None else None
@@ -1173,8 +1294,8 @@ class HipOps:
             raise KernelError(f"attention kernels: head size {dh} is not supported (a multiple of 8, at most 256)")
         if hq % hk:
             raise KernelError(f"attention kernels: {hq} query heads are no multiple of {hk} kv heads")
-        if (q.dtype == torch.float32 and dh % 16 == 0 and ps % 16 == 0 and n * hq >= self.GENERIC_SPLIT_BELOW
-                and (meta is None or meta.decode_bucket is None)):
+        if (not biased and q.dtype == torch.float32 and dh % 16 == 0 and ps % 16 == 0
+                and n * hq >= self.GENERIC_SPLIT_BELOW and (meta is None or meta.decode_bucket is None)):
             # many tokens in float32: tiles of 16 tokens on the float32 matrix instructions
             tiles = meta.meta.get("f32_tiles") if meta is not None else None
             if tiles is None:
@@ -1191,7 +1312,7 @@ class HipOps:
                        _p(block_table), block_table.shape[1], _p(tiles), tiles.numel() // 2, mode, param, float(scale),
                        hq, hk, dh, ps)
             return out
-        if (q.dtype == torch.float32 and dh % 16 == 0 and ps % 16 == 0 and hq // hk <= 16
+        if (not biased and q.dtype == torch.float32 and dh % 16 == 0 and ps % 16 == 0 and hq // hk <= 16
                 and ((meta is not None and meta.decode_bucket is not None)
                      or all(ln == 1 for ln in self._segments(meta, token_segment, positions)[0]))):
             # a step of single tokens in float32: the query heads of a kv head share a wavefront (its keys and
@@ -1231,6 +1352,12 @@ class HipOps:
                 splits = -(-tiles // tiles_per_split)
                 ws_ml = torch.empty(waves * splits * 2, dtype=torch.float32, device=q.device)
                 ws_o = torch.empty(waves * splits * dh, dtype=torch.float32, device=q.device)
+        if biased:
+            self._call("jle_paged_attention_biased", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
+                       _p(block_table), block_table.shape[1], mode, param, float(scale), self._is_bf16(q), n, hq, hk,
+                       dh, ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o), _p(bias),
+                       0 if bias is None else bias.shape[1], _p(sink))
+            return out
         self._call("jle_paged_attention_generic", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                    _p(block_table), block_table.shape[1], mode, param, float(scale), self._is_bf16(q), n, hq, hk, dh,
                    ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o))
@@ -1331,9 +1458,28 @@ class HipOps:
                    m, num_experts, k, int(extra_group))
         return offsets, sorted_token, sorted_gate, inv
 
+    def row_gate_(self, rows, h32, w):
+        """``rows[n] *= sigmoid(h32[n] . w)`` in place: one number a token, formed in float32."""
+        n, d = rows.shape
+        k = h32.shape[1]
+        self._chk(rows, None, (n, d), "rows")
+        self._chk(h32, torch.float32, (n, k), "gate input")
+        self._chk(w, torch.float32, None, "gate row")
+        if w.numel() != k:
+            raise KernelError("the gate's row does not fit its input")
+        self._call("jle_row_gate", _p(rows), self._is_bf16(rows), _p(h32), _p(w), n, k, d)
+        return rows
+
     def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None,
-                    shared_weights=None):
-        """``shared``: a shared expert's output, or ``shared_weights``: its (gate|up, down) matrices, row-major."""
+                    shared_weights=None, shared_gate=None):
+        """``shared``: a shared expert's output, or ``shared_weights``: its (gate|up, down) matrices, row-major.
+        ``shared_gate = (h32, w)``: the shared expert's output times ``sigmoid(h32 . w)``, one number a token."""
+        if shared_gate is not None:
+            total = self.moe_experts(h, expert_ids, gates, w_gate_up, w_down, shared=shared, tiled=tiled,
+                                     grouping=grouping, shared_weights=shared_weights)
+            if total.shared is not None:
+                self.row_gate_(total.shared, self._rows(shared_gate[0], want32=True), shared_gate[1])
+            return total
         h = self._rows(h)
         n, d = h.shape
         e, f2, _ = w_gate_up.shape
