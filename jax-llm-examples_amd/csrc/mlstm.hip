@@ -53,7 +53,9 @@ __device__ __forceinline__ float sum_over_p(float v) {
   return v;
 }
 
-template <typename T, int KP>
+// VEC: dv is a multiple of 4 (a lane's four columns are there together, and rows of q | k | v | gate and of the state
+// can be read four elements at a time); without it every column is guarded and read on its own.
+template <typename T, int KP, bool VEC>
 __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ rows, const float* __restrict__ gates,
                                                         float* __restrict__ state, const int* __restrict__ cu,
                                                         const int* __restrict__ slots, const int* __restrict__ phase,
@@ -62,7 +64,7 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ ro
   const int seg = blockIdx.x, h = blockIdx.y, slice = blockIdx.z;
   const int lane = threadIdx.x, p = lane >> 3, j4 = lane & 7;
   const int col = slice * 32 + 4 * j4;  // this lane's first value column
-  const bool col_ok = col < dv;         // (dv is a multiple of 4)
+  const bool col_ok = col < dv;
   const int t0 = cu[seg], t1 = cu[seg + 1];
   const int width = 2 * H * dk + 2 * H * dv;
   const size_t per_head = (size_t)dk * dv + dk + 1;
@@ -75,7 +77,16 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ ro
 #pragma unroll
   for (int i = 0; i < KP; ++i) {
     const int k = p + 8 * i;
-    C[i] = (k < dk && col_ok) ? *reinterpret_cast<const f32x4*>(st_in + (size_t)k * dv + col) : f32x4{0.f, 0.f, 0.f, 0.f};
+    C[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (k < dk && col_ok) {
+      if (VEC) {
+        C[i] = *reinterpret_cast<const f32x4*>(st_in + (size_t)k * dv + col);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (col + c < dv) C[i][c] = st_in[(size_t)k * dv + col + c];
+      }
+    }
     nn[i] = k < dk ? st_in[(size_t)dk * dv + k] : 0.f;
   }
   float m = st_in[(size_t)dk * dv + dk];
@@ -91,7 +102,16 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ ro
       qn[i] = k < dk ? Num<T>::load(r + h * dk + k) : 0.f;
       kn[i] = k < dk ? Num<T>::load(r + H * dk + h * dk + k) : 0.f;
     }
-    vn = col_ok ? load_v4<T>(r + 2 * H * dk + h * dv + col) : f32x4{0.f, 0.f, 0.f, 0.f};
+    vn = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (col_ok) {
+      if (VEC) {
+        vn = load_v4<T>(r + 2 * H * dk + h * dv + col);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (col + c < dv) vn[c] = Num<T>::load(r + 2 * H * dk + h * dv + col + c);
+      }
+    }
     gi = gates[(size_t)t * 2 * H + h];
     gf = gates[(size_t)t * 2 * H + H + h];
   };
@@ -133,13 +153,28 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ ro
     const float den = fmaxf(fabsf(nq), expf(-m)) + floor_;
     if (p == 0 && col_ok) {
       const f32x4 r = {o[0] / den, o[1] / den, o[2] / den, o[3] / den};
-      *reinterpret_cast<f32x4*>(o_raw + (size_t)t * H * dv + h * dv + col) = r;
+      float* dst = o_raw + (size_t)t * H * dv + h * dv + col;
+      if (VEC) {
+        *reinterpret_cast<f32x4*>(dst) = r;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (col + c < dv) dst[c] = r[c];
+      }
     }
   }
 #pragma unroll
   for (int i = 0; i < KP; ++i) {
     const int k = p + 8 * i;
-    if (k < dk && col_ok) *reinterpret_cast<f32x4*>(st_out + (size_t)k * dv + col) = C[i];
+    if (k < dk && col_ok) {
+      if (VEC) {
+        *reinterpret_cast<f32x4*>(st_out + (size_t)k * dv + col) = C[i];
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (col + c < dv) st_out[(size_t)k * dv + col + c] = C[i][c];
+      }
+    }
     if (k < dk && slice == 0 && j4 == 0) st_out[(size_t)dk * dv + k] = nn[i];
   }
   if (slice == 0 && lane == 0) st_out[(size_t)dk * dv + dk] = m;
@@ -171,7 +206,7 @@ JLE_API int jle_mlstm(const void* rows, int is_bf16, float* gates, const float* 
                       float* state, const int* cu, const int* slots, const int* phase, float* o_raw, void* out, int N,
                       int R, int H, int dk, int dv, float cap, float eps, float floor_, hipStream_t s) {
   if (N <= 0 || R <= 0) return 0;
-  if (H < 1 || dk < 1 || dk > 256 || dv < 4 || dv % 4 || !(cap > 0.f)) return JLE_BAD_ARG;
+  if (H < 1 || dk < 1 || dk > 256 || dv < 1 || !(cap > 0.f)) return JLE_BAD_ARG;
   const long long total = (long long)N * 2 * H;
   hipLaunchKernelGGL(mlstm_gates_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gates, b_gates, cap, H,
                      total);
@@ -179,9 +214,16 @@ JLE_API int jle_mlstm(const void* rows, int is_bf16, float* gates, const float* 
   const dim3 grid(R, H, (dv + 31) / 32);
   const float q_mul = 1.0f / sqrtf((float)dk);
   const int need = (dk + 7) / 8;
-#define SCAN(T, KP)                                                                                              \
-  hipLaunchKernelGGL((mlstm_scan_kernel<T, KP>), grid, dim3(64), 0, s, (const T*)rows, gates, state, cu, slots,  \
-                     phase, o_raw, H, dk, dv, q_mul, floor_)
+  const bool vec = dv % 4 == 0;
+#define SCAN(T, KP)                                                                                                   \
+  do {                                                                                                                \
+    if (vec)                                                                                                          \
+      hipLaunchKernelGGL((mlstm_scan_kernel<T, KP, true>), grid, dim3(64), 0, s, (const T*)rows, gates, state, cu,    \
+                         slots, phase, o_raw, H, dk, dv, q_mul, floor_);                                              \
+    else                                                                                                              \
+      hipLaunchKernelGGL((mlstm_scan_kernel<T, KP, false>), grid, dim3(64), 0, s, (const T*)rows, gates, state, cu,   \
+                         slots, phase, o_raw, H, dk, dv, q_mul, floor_);                                              \
+  } while (0)
 #define PICK(T)                   \
   do {                            \
     if (need <= 2) SCAN(T, 2);    \

@@ -328,8 +328,8 @@ class HipOps:
         self._chk(ctx.state_phase, torch.int32, (r,), "state phases")
         if ctx.num_tokens != n:
             raise KernelError("the rows do not fit the step")
-        if dv % 4 or dk > 256:
-            raise KernelError(f"matrix-memory kernel: value size {dv} must be a multiple of 4 and key size {dk} at most 256")
+        if dk > 256:
+            raise KernelError(f"matrix-memory kernel: key size {dk} must be at most 256")
         o_raw = torch.empty(n, H * dv, dtype=torch.float32, device=rows.device)
         out = torch.empty(n, H * dv, dtype=rows.dtype, device=rows.device)
         self._call("jle_mlstm", _p(rows), self._is_bf16(rows), _p(gates), _p(b_gates), _p(norm_weight), _p(state),

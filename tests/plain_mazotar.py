@@ -75,7 +75,8 @@ def biased_sink_attention(h, w, prefix, m, eps, positions, keys, values):
     T = h.shape[0]
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = weighted_norm(h @ w[prefix + "q"].T, w[prefix + "q.norm"], eps)
-    temp = torch.tensor([query_temperature(p, m["q_temp"]["coef"], m["q_temp"]["every"]) for p in positions],
+    qt = m.get("q_temp")  # (absent: no temperature)
+    temp = torch.tensor([1.0 if qt is None else query_temperature(p, qt["coef"], qt["every"]) for p in positions],
                         dtype=h.dtype)
     q = (q * temp[:, None]).view(T, H, dk)
     k, v = keys.view(T, G, dk), values.view(T, G, dv)
