@@ -66,7 +66,30 @@ def design_configs(size: dict, layers: int):
                            "mlp": {"kind": "dense", "ff": size["ff"]}} for i in range(layers)]}
     if layers >= 3:
         tiradra["loop"] = {"start": 1, "stop": layers - 1, "times": 2}
-    return {"rovidra": rovidra, "tiradra": tiradra, "llama4-dense": llama}
+    # Mazotar: a matrix-memory layer and an attention layer (distance table, sinks, norms over the projections) in
+    # turn, every second attention layer on the keys and values of the one before it, four residual streams, eight
+    # experts of half the feed-forward width (one a token) beside a gated shared one; and the closest model the
+    # engine has for it: Llama 4 with routed layers of the same experts
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 1}, "expert": {"ff": size["ff"] // 2},
+           "shared": {"ff": size["ff"] // 2}}
+    m_attn = {"heads": size["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "bias_max": 128,
+              "bias_rows": 32, "q_temp": {"coef": 0.1, "every": 8192}}
+    m_mem = {"heads": size["heads"], "dim": 64, "vdim": 128, "gate_cap": 15.0}
+    m_layers, last_attn = [], None
+    for i in range(layers):
+        if i % 2 == 0:
+            m_layers.append({"type": "mlstm", "mixer": m_mem, "mlp": moe})
+        elif last_attn is None:
+            m_layers.append({"type": "attention", "mixer": m_attn, "mlp": moe})
+            last_attn = i
+        else:
+            m_layers.append({"type": "attention", "mixer": dict(m_attn, kv_from=last_attn), "mlp": moe})
+            last_attn = None
+    mazotar = {"architecture": "Mazotar", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-5},
+               "embedding": {"scale": 1.0}, "streams": 4, "layers": m_layers}
+    llama_moe = dict(llama, interleave_moe_layer_step=1, moe_layers=list(range(layers)), num_local_experts=8,
+                     num_experts_per_tok=1, intermediate_size=size["ff"] // 2)
+    return {"rovidra": rovidra, "tiradra": tiradra, "llama4-dense": llama, "mazotar": mazotar, "llama4-moe": llama_moe}
 
 
 def bench_designs(args) -> int:
@@ -174,10 +197,11 @@ def main() -> int:
     ap.add_argument("--preset", default="llama4-scout")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--design-points", default="1@2048,8@2048,64@2048", help="decode steps of --designs: batch@context")
-    ap.add_argument("--designs", default="", help="instead of the default workload: prefill and decode of the Rovidra "
-                    "and Tiradra designs beside the dense Llama 4 layer of equal sizes, at the named sizes "
+    ap.add_argument("--designs", default="", help="instead of the default workload: prefill and decode of the Rovidra, "
+                    "Tiradra and Mazotar designs beside the Llama 4 layers of equal sizes, at the named sizes "
                     "(comma-separated, of " + ", ".join(DESIGN_SIZES) + "; 'all')")
-    ap.add_argument("--design-names", default="", help="with --designs: only these of rovidra, tiradra, llama4-dense")
+    ap.add_argument("--design-names", default="", help="with --designs: only these of rovidra, tiradra, llama4-dense, "
+                    "mazotar, llama4-moe")
     args = ap.parse_args()
     if args.designs:
         return bench_designs(args)
