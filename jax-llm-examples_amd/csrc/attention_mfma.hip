@@ -48,6 +48,13 @@ struct Columns {  // per lane, for each of its column tiles
   int token;      // row of q / out
   int head;       // query head
   int lo, hi;     // keys this column may read within the wave's range (inclusive); lo > hi: none
+  int pos;        // the query's position (read by the kernels that add a distance bias only)
+};
+
+// A learned number per (query head, distance) added to the scaled score: table[h][min(pos - key, L - 1)], float32.
+struct Biasing {
+  const float* table;
+  int L;
 };
 
 // Maximum / sum over the four lanes that hold one column (equal lane % 16), in all of them.  The two swaps
@@ -77,14 +84,22 @@ __device__ __forceinline__ float column_sum(float v) {
 //   st[ct][tt]: scores of key tile tt (keys kb + 16 tt + 4 g + i in element i); act0 / act1: the tile exists
 //   vraw[dt]: for element row 16 dt + (lane % 16): keys 4 g .. 4 g + 3 of tile 0 (x, y) and of tile 1 (z, w)
 //   l: each lane's own part of the column's sum (column_sum at the end gives the whole)
-template <int DH, int CT, bool MASKED, typename V4>
+//   BIASED: a distance bias is added to every scaled score (far: every key of the step is so far behind every
+//   live column that the table's last entry holds, far_b[ct], already in the exponent's base-2 units), and the
+//   probabilities enter the second product as two bfloat16 terms (leading part and remainder) instead of one
+//   rounded term, which keeps about 16 bits of them.
+template <int DH, int CT, bool MASKED, typename V4, bool BIASED = false>
 __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], bool act0, bool act1,
                                                    const V4 (&vraw)[DH / 16], int kb, const Columns (&col)[CT],
                                                    int k_lo, int k_hi, float scale_log2, float (&m)[CT],
-                                                   float (&l)[CT], f32x4 (&acc)[CT][DH / 16]) {
+                                                   float (&l)[CT], f32x4 (&acc)[CT][DH / 16],
+                                                   Biasing bias = Biasing{nullptr, 0}, bool far = false,
+                                                   const float* far_b = nullptr) {
   constexpr int DT = DH / 16;
   const int g = (threadIdx.x & 63) >> 4;
+  const float sc = BIASED ? 1.0f : scale_log2;  // (biased scores are scaled where the bias is added)
   bf16x8 pb[CT];
+  bf16x8 pb_lo[BIASED ? CT : 1];
   float corr[CT];
   bool unchanged = true;
 #pragma unroll
@@ -96,6 +111,14 @@ __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], boo
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float v = st[ct][tt][i];
+        if (BIASED) {
+          float b = far_b[ct];
+          if (!far) {
+            const int back = col[ct].pos - (kb + 16 * tt + 4 * g + i);
+            b = bias.table[(size_t)col[ct].head * bias.L + min(max(back, 0), bias.L - 1)] * kLog2e;
+          }
+          v = fmaf(v, scale_log2, b);
+        }
         if (MASKED) {
           const int key = kb + 16 * tt + 4 * g + i;
           const bool ok = (tt == 0 ? act0 : act1) && key >= col[ct].lo && key <= col[ct].hi;
@@ -105,7 +128,7 @@ __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], boo
         mx = fmaxf(mx, v);
       }
     mx = column_max(mx);
-    const float m_new = fmaxf(m[ct], mx * scale_log2);  // the scale is positive
+    const float m_new = fmaxf(m[ct], mx * sc);  // the scale is positive
     const float m_use = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
     corr[ct] = __builtin_amdgcn_exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
     unchanged = unchanged && m_new == m[ct];
@@ -113,13 +136,24 @@ __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], boo
     float p[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      p[j] = __builtin_amdgcn_exp2f(fmaf(s[j], scale_log2, -m_use));  // masked: exp2(-inf) = 0
+      p[j] = __builtin_amdgcn_exp2f(fmaf(s[j], sc, -m_use));  // masked: exp2(-inf) = 0
       sum += p[j];
     }
     l[ct] = l[ct] * corr[ct] + sum;
     m[ct] = m_new;
     const uint4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
     pb[ct] = __builtin_bit_cast(bf16x8, pk);
+    if (BIASED) {  // what the rounding left out, as a second term
+      float r[8];
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        const uint32_t w = j == 0 ? pk.x : j == 2 ? pk.y : j == 4 ? pk.z : pk.w;
+        r[j] = p[j] - __uint_as_float(w << 16);
+        r[j + 1] = p[j + 1] - __uint_as_float(w & 0xffff0000u);
+      }
+      const uint4 rk = {pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]), pack_bf16(r[4], r[5]), pack_bf16(r[6], r[7])};
+      pb_lo[ct] = __builtin_bit_cast(bf16x8, rk);
+    }
   }
   // no column of the wavefront has a new maximum: every factor is exactly one (or the sums are still zero)
   if (!__all(unchanged)) {
@@ -155,16 +189,20 @@ __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], boo
       vv.w &= keep[1][1];
       const bf16x8 a = __builtin_bit_cast(bf16x8, vv);
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CT; ++ct) {
+        if (BIASED) acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb_lo[ct], acc[ct][dt], 0, 0, 0);
         acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
+      }
     }
   } else {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       const bf16x8 a = __builtin_bit_cast(bf16x8, vraw[dt]);
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CT; ++ct) {
+        if (BIASED) acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb_lo[ct], acc[ct][dt], 0, 0, 0);
         acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
+      }
     }
   }
 }
@@ -214,11 +252,12 @@ __device__ __forceinline__ void load_queries(const bf16_t* __restrict__ q, const
   }
 }
 
-template <int DH, int CT, bool ONCE>
+template <int DH, int CT, bool ONCE, bool BIASED = false>
 __device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], const bf16_t* __restrict__ kv,
                                             const int* __restrict__ table, const Columns (&col)[CT], int k_lo,
                                             int k_hi, int hk, int Hkv, int ps, float scale_log2, float (&m)[CT],
-                                            float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad) {
+                                            float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad,
+                                            Biasing bias = Biasing{nullptr, 0}) {
   const int lane = threadIdx.x & 63;
   const int c16 = lane & 15, g = lane >> 4;
   constexpr int KC = DH / 32;  // k-steps of the first product
@@ -301,6 +340,21 @@ __device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], con
   };
   int all_lo, all_hi;
   common_range<CT>(col, all_lo, all_hi);
+  // with a distance bias: the table's last entry per column, and the last key that is that far behind every
+  // live column of the wavefront
+  float far_b[CT];
+  int far_until = INT_MIN;
+  if (BIASED) {
+    int min_pos = INT_MAX;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      far_b[ct] = bias.table[(size_t)col[ct].head * bias.L + bias.L - 1] * kLog2e;
+      if (col[ct].lo <= col[ct].hi) min_pos = min(min_pos, col[ct].pos);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) min_pos = min(min_pos, __shfl_xor(min_pos, o, 64));
+    far_until = min_pos == INT_MAX ? INT_MIN : min_pos - (bias.L - 1);
+  }
   look_up();
   if (kb_first <= k_hi) load_step();
   for (int kb = kb_first; kb <= k_hi; kb += 32) {
@@ -324,6 +378,16 @@ __device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], con
     }
     // the next step's keys and values (this step keeps act0 / act1 and vraw)
     if (kb + 32 <= k_hi) load_step();
+    if (BIASED) {
+      const bool far = kb + 31 <= far_until;
+      if (__all(act0 && act1 && kb >= all_lo && kb + 31 <= all_hi))
+        softmax_and_values<DH, CT, false, u32x4, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l,
+                                                       acc, bias, far, far_b);
+      else
+        softmax_and_values<DH, CT, true, u32x4, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l,
+                                                      acc, bias, far, far_b);
+      continue;
+    }
     if (__all(act0 && act1 && kb >= all_lo && kb + 31 <= all_hi))
       softmax_and_values<DH, CT, false>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
     else
@@ -333,26 +397,29 @@ __device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], con
   for (int ct = 0; ct < CT; ++ct) l[ct] = column_sum(l[ct]);
 }
 
-template <int DH, int CT, bool ONCE>
+template <int DH, int CT, bool ONCE, bool BIASED = false>
 __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv,
                                        const int* __restrict__ table, const Columns (&col)[CT], int k_lo, int k_hi,
                                        int hk, int Hq, int Hkv, int ps, float scale_log2, float (&m)[CT],
-                                       float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad) {
+                                       float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad,
+                                       Biasing bias = Biasing{nullptr, 0}) {
   bf16x8 qb[CT][DH / 32];
   load_queries<DH, CT>(q, col, Hq, qb);
-  attend_with<DH, CT, ONCE>(qb, kv, table, col, k_lo, k_hi, hk, Hkv, ps, scale_log2, m, l, acc, bad);
+  attend_with<DH, CT, ONCE, BIASED>(qb, kv, table, col, k_lo, k_hi, hk, Hkv, ps, scale_log2, m, l, acc, bad, bias);
 }
 
 // ------------------------------------------------------------------ prefill portions
 // tiles: [num_tiles][2] = (first token, number of tokens <= 16 * CT), all of one segment.
 // One wavefront per (tile, query head); the heads of one kv head are neighbours.
 // (launch bounds: with one column tile and head sizes up to 128 the registers are held to what lets two wavefronts share a SIMD)
-template <int DH, int CT>
-__global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention_prefill_kernel(
+// BIASED: a distance bias (see Biasing) on every score and, with `sink`, one more term exp(sink[h]) in head h's
+// denominator.
+template <int DH, int CT, bool BIASED = false>
+__global__ __launch_bounds__(256, (CT == 1 && DH <= 128 && !BIASED) ? 2 : 1) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ tiles, int num_tiles, int ret_mode, int ret_param, float scale_log2,
-    int Hq, int Hkv, int ps) {
+    int Hq, int Hkv, int ps, Biasing bias = Biasing{nullptr, 0}, const float* __restrict__ sink = nullptr) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave_index();
   if (item >= num_tiles * Hq) return;
@@ -374,16 +441,18 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
     col[ct].head = h;
     col[ct].lo = ok ? first_key(ret_mode, ret_param, pos) : 1;
     col[ct].hi = ok ? pos : 0;
+    col[ct].pos = pos;
   }
   float m[CT], l[CT];
   f32x4 acc[CT][DH / 16];
   bool bad = false;
-  attend<DH, CT, false>(q, kv, block_table + (size_t)token_segment[n0] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
-                 scale_log2, m, l, acc, bad);
+  attend<DH, CT, false, BIASED>(q, kv, block_table + (size_t)token_segment[n0] * table_width, col, k_lo, k_hi, hk, Hq,
+                                Hkv, ps, scale_log2, m, l, acc, bad, bias);
   bad = __any(bad);
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     if (ct * 16 + c16 >= nt) continue;
+    if (BIASED && sink != nullptr) l[ct] += exp2f(sink[h] * kLog2e - m[ct]);
     const float inv = bad ? __builtin_nanf("") : (l[ct] > 0.f ? 1.0f / l[ct] : 0.f);
     bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
 #pragma unroll
@@ -958,12 +1027,12 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
 // dec_tokens: [num_dec] rows of q that are single decode tokens.  One wavefront per
 // (decode token, kv head, key range); ws_ml: [item][16 * CT][2], ws_o: [item][16 * CT][DH],
 // item = (d * Hkv + hk) * max_splits + split.
-template <int DH, int CT>
-__global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention_decode_kernel(
+template <int DH, int CT, bool BIASED = false>
+__global__ __launch_bounds__(256, (CT == 1 && DH <= 128 && !BIASED) ? 2 : 1) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, float* __restrict__ ws_ml, float* __restrict__ ws_o,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ dec_tokens, int num_dec, int max_splits, int kSplit, int ret_mode,
-    int ret_param, float scale_log2, int Hq, int Hkv, int ps) {
+    int ret_param, float scale_log2, int Hq, int Hkv, int ps, Biasing bias = Biasing{nullptr, 0}) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave_index();
   if (item >= num_dec * Hkv * max_splits) return;
@@ -987,12 +1056,13 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
     col[ct].head = ok ? hk * G + c : hk * G;
     col[ct].lo = ok ? k_lo : 1;
     col[ct].hi = ok ? k_hi : 0;
+    col[ct].pos = pos;
   }
   float m[CT], l[CT];
   f32x4 acc[CT][DH / 16];
   bool bad = false;
-  attend<DH, CT, true>(q, kv, block_table + (size_t)token_segment[n] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
-                 scale_log2, m, l, acc, bad);
+  attend<DH, CT, true, BIASED>(q, kv, block_table + (size_t)token_segment[n] * table_width, col, k_lo, k_hi, hk, Hq,
+                               Hkv, ps, scale_log2, m, l, acc, bad, bias);
   bad = __any(bad);
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
@@ -1015,7 +1085,8 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
 __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
                                               bf16_t* __restrict__ out, const int* __restrict__ positions,
                                               const int* __restrict__ dec_tokens, int max_splits, int kSplit,
-                                              int ret_mode, int ret_param, int Hq, int Hkv, int DH, int cols) {
+                                              int ret_mode, int ret_param, int Hq, int Hkv, int DH, int cols,
+                                              const float* __restrict__ sink) {
   __shared__ float red_max[4], red_sum[4];
   __shared__ int red_nan[4];
   const int d = blockIdx.x / Hq, h = blockIdx.x % Hq;
@@ -1060,6 +1131,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, c
   __syncthreads();
   l = red_sum[0];
   for (int w = 1; w < waves; ++w) l += red_sum[w];
+  if (sink != nullptr) l += exp2f(sink[h] * kLog2e - mx);  // one more term of the denominator, once
 
   for (int e = threadIdx.x; e < DH; e += blockDim.x) {
     float o = 0.f;
@@ -1368,9 +1440,14 @@ JLE_API int jle_attention_mfma_supported(int dh, int Hq, int Hkv, int ps) {
 JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, const int* positions,
                                   const int* token_segment, const int* block_table, int table_width, const int* tiles,
                                   int num_tiles, int tile_tokens, const int* groups, int num_groups, int ret_mode,
-                                  int ret_param, float scale, int Hq, int Hkv, int dh, int ps, hipStream_t s) {
+                                  int ret_param, float scale, int Hq, int Hkv, int dh, int ps, const float* bias,
+                                  int bias_len, const float* sink, hipStream_t s) {
   if (num_tiles <= 0) return 0;
   if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps)) return JLE_BAD_ARG;
+  // bias: [Hq][bias_len] (with a sink and no bias: a table of zeros); the kernels that share keys take neither
+  if ((bias == nullptr) != (bias_len == 0) || (sink != nullptr && bias == nullptr)) return JLE_BAD_ARG;
+  if (bias != nullptr && groups != nullptr) return JLE_BAD_ARG;
+  const Biasing bs = {bias, bias_len};
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
   const long long items = (long long)num_tiles * Hq;
   dim3 g((unsigned)((items + 3) / 4)), b(256);
@@ -1400,16 +1477,19 @@ JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, cons
     JLE_LAUNCH_CHECK();
     return 0;
   }
+#define LAUNCH_B(DH, CT, BIASED)                                                                                     \
+  hipLaunchKernelGGL((attention_prefill_kernel<DH, CT, BIASED>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,    \
+                     (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles, ret_mode,   \
+                     ret_param, sl, Hq, Hkv, ps, bs, sink)
 #define LAUNCH(DH)                                                                                                   \
   do {                                                                                                               \
-    if (tile_tokens == 32)                                                                                           \
-      hipLaunchKernelGGL((attention_prefill_kernel<DH, 2>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,         \
-                         (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles,         \
-                         ret_mode, ret_param, sl, Hq, Hkv, ps);                                                      \
-    else                                                                                                             \
-      hipLaunchKernelGGL((attention_prefill_kernel<DH, 1>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,         \
-                         (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles,         \
-                         ret_mode, ret_param, sl, Hq, Hkv, ps);                                                      \
+    if (tile_tokens == 32) {                                                                                         \
+      if (bias != nullptr) LAUNCH_B(DH, 2, true);                                                                    \
+      else LAUNCH_B(DH, 2, false);                                                                                   \
+    } else {                                                                                                         \
+      if (bias != nullptr) LAUNCH_B(DH, 1, true);                                                                    \
+      else LAUNCH_B(DH, 1, false);                                                                                   \
+    }                                                                                                                \
   } while (0)
   switch (dh) {
     case 32: LAUNCH(32); break;
@@ -1419,6 +1499,7 @@ JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, cons
     case 256: LAUNCH(256); break;
   }
 #undef LAUNCH
+#undef LAUNCH_B
   JLE_LAUNCH_CHECK();
   return 0;
 }
@@ -1428,9 +1509,11 @@ JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float
                                  const int* positions, const int* token_segment, const int* block_table,
                                  int table_width, const int* dec_tokens, int num_dec, int max_splits, int split,
                                  int ret_mode, int ret_param, float scale, int Hq, int Hkv, int dh, int ps,
-                                 hipStream_t s) {
+                                 const float* bias, int bias_len, const float* sink, hipStream_t s) {
   if (num_dec <= 0) return 0;
   if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps) || max_splits < 1 || split < 32 || split % 32) return JLE_BAD_ARG;
+  if ((bias == nullptr) != (bias_len == 0) || (sink != nullptr && bias == nullptr)) return JLE_BAD_ARG;
+  const Biasing bs = {bias, bias_len};
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
   const int G = Hq / Hkv;
   if (G > 32) return JLE_BAD_ARG;
@@ -1438,14 +1521,19 @@ JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float
   const long long items = (long long)num_dec * Hkv * max_splits;
   dim3 g((unsigned)((items + 3) / 4)), b(256);
   const float sl = scale * kLog2e;
-#define LAUNCH(DH, CT)                                                                                              \
-  hipLaunchKernelGGL((attention_decode_kernel<DH, CT>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv, ws_ml,     \
-                     ws_o, positions, token_segment, block_table, table_width, dec_tokens, num_dec, max_splits,     \
-                     split, ret_mode, ret_param, sl, Hq, Hkv, ps)
-#define PICK(DH)          \
-  do {                    \
-    if (ct == 1) LAUNCH(DH, 1); \
-    else LAUNCH(DH, 2);   \
+#define LAUNCH(DH, CT, BIASED)                                                                                      \
+  hipLaunchKernelGGL((attention_decode_kernel<DH, CT, BIASED>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,    \
+                     ws_ml, ws_o, positions, token_segment, block_table, table_width, dec_tokens, num_dec,          \
+                     max_splits, split, ret_mode, ret_param, sl, Hq, Hkv, ps, bs)
+#define PICK(DH)                             \
+  do {                                       \
+    if (bias != nullptr) {                   \
+      if (ct == 1) LAUNCH(DH, 1, true);      \
+      else LAUNCH(DH, 2, true);              \
+    } else {                                 \
+      if (ct == 1) LAUNCH(DH, 1, false);     \
+      else LAUNCH(DH, 2, false);             \
+    }                                        \
   } while (0)
   switch (dh) {
     case 32: PICK(32); break;
@@ -1458,7 +1546,8 @@ JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float
 #undef LAUNCH
   JLE_LAUNCH_CHECK();
   hipLaunchKernelGGL(attention_decode_merge_kernel, dim3(num_dec * Hq), dim3(dh <= 64 ? 64 : 128), 0, s, ws_ml, ws_o,
-                     (bf16_t*)out, positions, dec_tokens, max_splits, split, ret_mode, ret_param, Hq, Hkv, dh, 16 * ct);
+                     (bf16_t*)out, positions, dec_tokens, max_splits, split, ret_mode, ret_param, Hq, Hkv, dh, 16 * ct,
+                     sink);
   JLE_LAUNCH_CHECK();
   return 0;
 }

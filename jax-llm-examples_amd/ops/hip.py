@@ -49,9 +49,10 @@ _SIGNATURES = {
     "jle_gemm_f32_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
-    "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
+    "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp,
+                              _i, _vp, _vp],
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
-                             _vp],
+                             _vp, _i, _vp, _vp],
     "jle_attention_decode_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i,
                                    _i, _i, _vp, _f, _f, _f, _vp, _i, _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -185,6 +186,7 @@ class HipOps:
         # counters of the kernels in which the last wavefront (or block) to finish does the closing work: zero
         # between launches (whoever closes puts its counter back), so they are cleared here once
         self._tickets = torch.zeros(self.TICKETS, dtype=torch.int32, device=self.device)
+        self._zero_bias = {}  # (heads, device) -> a distance table of zeros, for sinks without a bias
         self._slice_tickets = torch.zeros(self.SLICE_TICKETS, dtype=torch.int32, device=self.device)
         self._compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         torch.backends.cuda.matmul.allow_tf32 = False
@@ -1266,13 +1268,20 @@ class HipOps:
             self._chk(bias, torch.float32, (hq, bias.shape[1]), "distance bias")
         if sink is not None:
             self._chk(sink, torch.float32, (hq,), "sinks")
-        if (not biased and q.dtype == torch.bfloat16 and hq // hk <= 32
+        if (q.dtype == torch.bfloat16 and hq // hk <= 32
                 and self._query("jle_attention_mfma_supported", dh, hq, hk, ps)):
-            key = f"attn_plan_{hq // hk}"
+            # (with a bias or sinks: every (tile, head) a wavefront of its own, no keys shared between wavefronts)
+            grouped = 1 if biased else hq // hk
+            if biased and bias is None:
+                bias = self._zero_bias.get((hq, q.device))
+                if bias is None:
+                    bias = self._zero_bias[(hq, q.device)] = torch.zeros(hq, 1, dtype=torch.float32, device=q.device)
+            bias_len = bias.shape[1] if biased else 0
+            key = f"attn_plan_{grouped}"
             plan = meta.meta.get(key) if meta is not None else None
             if plan is None:
                 seg_lens, seg_starts = self._segments(meta, token_segment, positions)
-                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk, hq // hk,
+                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk, grouped,
                                            decode_bucket=meta.decode_bucket if meta is not None else None)
                 if meta is not None:
                     meta.meta[key] = plan
@@ -1280,7 +1289,7 @@ class HipOps:
                 self._call("jle_attention_prefill", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                            _p(block_table), block_table.shape[1], _p(plan["tiles"]), plan["num_tiles"],
                            self.PREFILL_TILE, _p(plan["groups"]), plan["num_groups"], mode, param, float(scale), hq,
-                           hk, dh, ps)
+                           hk, dh, ps, _p(bias), bias_len, _p(sink))
             if plan["num_dec"]:
                 cols = 16 if hq // hk <= 16 else 32
                 items = plan["num_dec"] * hk * plan["max_splits"]
@@ -1288,7 +1297,8 @@ class HipOps:
                 ws_o = torch.empty(items * cols * dh, dtype=torch.float32, device=q.device)
                 self._call("jle_attention_decode", _p(q), _p(kv_cache), _p(out), _p(ws_ml), _p(ws_o), _p(positions),
                            _p(token_segment), _p(block_table), block_table.shape[1], _p(plan["dec"]), plan["num_dec"],
-                           plan["max_splits"], plan["split"], mode, param, float(scale), hq, hk, dh, ps)
+                           plan["max_splits"], plan["split"], mode, param, float(scale), hq, hk, dh, ps, _p(bias),
+                           bias_len, _p(sink))
             return out
         if dh % 8 or dh > 256:
             raise KernelError(f"attention kernels: head size {dh} is not supported (a multiple of 8, at most 256)")

@@ -271,6 +271,61 @@ def test_paged_attention_of_long_portions_at_head_size_128(ops, ref, hq, hk, ps,
     _assert_close_to_scale(got, want, dt)
 
 
+def _distance_table(hq, length, seed):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(hq, length, generator=g) * 1.5).to(DEV)
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("hq,hk,dh,ps", [(4, 2, 16, 16), (8, 2, 64, 16), (10, 2, 128, 16), (5, 1, 96, 48), (3, 3, 32, 32),
+                                         (34, 2, 32, 16), (2, 1, 256, 16), (6, 3, 80, 16)])
+@pytest.mark.parametrize("length,with_sink", [(1, True), (9, True), (41, False), (130, True), (700, True)])
+def test_attention_with_distance_bias_and_sinks(ops, ref, monkeypatch, dt, hq, hk, dh, ps, length, with_sink):
+    """Portions and single tokens in one step, with a table that ends before, inside and beyond the contexts, keys
+    ranges of a single token that are merged, and a sink per head that is larger or smaller than the scores."""
+    specs = [(0, 70), (130, 1), (45, 9), (63, 2), (200, 1), (600, 1), (255, 35), (0, 1)]
+    q, kv, bt, pos, seg = _attention_case(hq, hk, dh, ps, dt, specs, seed=2)
+    bias = _distance_table(hq, length, seed=length)
+    sink = (torch.linspace(-6.0, 7.0, hq)).to(DEV) if with_sink else None
+    calls = []
+    inner = ops._call
+    monkeypatch.setattr(ops, "_call", lambda name, *a: (calls.append(name), inner(name, *a))[1])
+    got = ops.paged_attention(q, kv, bt, pos, seg, ("all",), dh ** -0.5, bias=bias, sink=sink)
+    if dt == torch.bfloat16 and dh in (32, 64, 96, 128, 256):
+        assert calls == ["jle_attention_prefill", "jle_attention_decode"]
+    want = ref.paged_attention(q, kv, bt, pos, seg, ("all",), dh ** -0.5, bias=bias, sink=sink)
+    _assert_close_to_scale(got, want, dt)
+    if with_sink:  # a sink alone
+        got = ops.paged_attention(q, kv, bt, pos, seg, ("all",), dh ** -0.5, sink=sink)
+        want = ref.paged_attention(q, kv, bt, pos, seg, ("all",), dh ** -0.5, sink=sink)
+        _assert_close_to_scale(got, want, dt)
+
+
+@pytest.mark.parametrize("dh", [64, 128])
+@pytest.mark.parametrize("back", [0, 1, 30, 31, 32, 63, 64, 65, 200])
+def test_a_distance_table_entry_that_stands_out_picks_its_key(ops, ref, dh, back):
+    """One entry of the table is so large that the key that many places back takes the whole weight, in a portion
+    and in a single token with merged key ranges; in the table's last entry every key from there on shares it.
+    With all queries zero the scores are the table's alone."""
+    dt = torch.bfloat16
+    hq, hk, ps, length = 4, 2, 16, 65
+    q, kv, bt, pos, seg = _attention_case(hq, hk, dh, ps, dt, [(100, 250), (2000, 1), (3, 40)], seed=4)
+    q = torch.zeros_like(q)
+    bias = torch.zeros(hq, length, device=DEV)
+    bias[:, min(back, length - 1)] = 60.0
+    got = ops.paged_attention(q, kv, bt, pos, seg, ("all",), dh ** -0.5, bias=bias).float().view(-1, hq, dh)
+    vt = kv[:, 1].reshape(kv.shape[0], hk, dh, ps).float()  # (the value planes lie transposed)
+    for i in (0, 17, 249, 250, 251, 290):
+        p, sg = int(pos[i]), int(seg[i])
+        firsts = [p - back] if back < length - 1 else list(range(0, p - length + 2))
+        firsts = [k for k in firsts if k >= 0]
+        if not firsts:
+            continue
+        rows = torch.stack([vt[int(bt[sg, k // ps]), :, :, k % ps] for k in firsts]).mean(dim=0)  # [hk, dh]
+        want = rows.repeat_interleave(hq // hk, dim=0)
+        assert torch.allclose(got[i], want, atol=2e-2), (i, back)
+
+
 def _decode_case(hq, hk, dh, ps, dt, contexts, seed=0):
     """One new token per request after ``contexts[i]`` tokens in the cache; the step's group context with the
     bound the kernels' work is laid out for; raw q|k|v rows and the slots of the new tokens."""
