@@ -83,6 +83,8 @@ _SIGNATURES = {
                              _vp],
     "jle_embed_sinusoid": [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _vp],
     "jle_mlstm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _f, _f, _vp],
+    "jle_mlstm_chunked": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
+                          _i, _i, _f, _f, _f, _vp],
     "jle_span_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_row_gate": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
     "jle_paged_attention_biased": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
@@ -147,7 +149,8 @@ def _bind(path: str):
             fn.restype = ctypes.c_int
     for name, args in (("jle_attention_mfma_supported", [_i, _i, _i, _i]),  # queries, not launches: no stream
                        ("jle_gemm_stream_supported", [_i, _i, _i]), ("jle_gemm_f32_stream_supported", [_i, _i, _i]),
-                       ("jle_latent_attention_mfma_supported", [_i, _i, _i, _i, _i]), ("jle_attention_group_waves", [])):
+                       ("jle_latent_attention_mfma_supported", [_i, _i, _i, _i, _i]), ("jle_attention_group_waves", []),
+                       ("jle_mlstm_chunked_supported", [_i, _i]), ("jle_mlstm_chunk_tokens", [])):
         fn = getattr(lib, name, None)
         if fn is not None:
             fn.argtypes = args
@@ -312,6 +315,8 @@ class HipOps:
         return out, out32
 
     # ------------------------------------------------------------------ a matrix memory per head
+    MLSTM_CHUNKS_FROM = 8  # a step with a segment of this many tokens takes the matrix memory in chunks
+
     def mlstm(self, rows, gates, b_gates, norm_weight, num_heads: int, head_dim: int, value_dim: int, cap: float,
               eps: float, floor: float, state, ctx):
         """``rows``: q | k | v | output gate in the run dtype; ``gates``: float32 ``[N, 2 H]`` pre-activations without
@@ -334,6 +339,29 @@ class HipOps:
             raise KernelError(f"matrix-memory kernel: key size {dk} must be at most 256")
         o_raw = torch.empty(n, H * dv, dtype=torch.float32, device=rows.device)
         out = torch.empty(n, H * dv, dtype=rows.dtype, device=rows.device)
+        if (max(ctx.seg_lens, default=0) >= self.MLSTM_CHUNKS_FROM
+                and self._query("jle_mlstm_chunked_supported", dk, dv)):
+            # a segment of many tokens: all segments in chunks that are worked on side by side
+            table = ctx.scratch.get("mlstm_chunks")
+            if table is None:
+                per = int(self._query("jle_mlstm_chunk_tokens"))
+                flat, firsts, o = [], [0], 0
+                for i, ln in enumerate(ctx.seg_lens):
+                    for t in range(0, ln, per):
+                        flat += [i, o + t, min(per, ln - t)]
+                    firsts.append(len(flat) // 3)
+                    o += ln
+                both = torch.tensor(flat + firsts, dtype=torch.int32).to(rows.device)
+                table = ctx.scratch["mlstm_chunks"] = (both[: len(flat)], both[len(flat):], len(flat) // 3)
+            chunks, seg_chunk0, nc = table
+            ws = torch.empty(nc * H * (dk * dv + dk + 3), dtype=torch.float32, device=rows.device)
+            ws_c, ws_n = ws[: nc * H * dk * dv], ws[nc * H * dk * dv: nc * H * (dk * dv + dk)]
+            ws_m, ws_m0 = ws[nc * H * (dk * dv + dk): nc * H * (dk * dv + dk + 2)], ws[nc * H * (dk * dv + dk + 2):]
+            self._call("jle_mlstm_chunked", _p(rows), self._is_bf16(rows), _p(gates), _p(b_gates), _p(norm_weight),
+                       _p(state), _p(ctx.state_slots), _p(ctx.state_phase), _p(chunks), nc, _p(seg_chunk0), _p(ws_c),
+                       _p(ws_n), _p(ws_m), _p(ws_m0), _p(o_raw), _p(out), n, r, H, dk, dv, float(cap), float(eps),
+                       float(floor))
+            return out
         self._call("jle_mlstm", _p(rows), self._is_bf16(rows), _p(gates), _p(b_gates), _p(norm_weight), _p(state),
                    _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(o_raw), _p(out), n, r, H, dk, dv,
                    float(cap), float(eps), float(floor))

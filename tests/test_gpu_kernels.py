@@ -271,6 +271,93 @@ def test_paged_attention_of_long_portions_at_head_size_128(ops, ref, hq, hk, ps,
     _assert_close_to_scale(got, want, dt)
 
 
+class _Segments:
+    """What the matrix-memory kernels read of a step."""
+
+    def __init__(self, seg_lens, slots, phases):
+        cu = [0]
+        for ln in seg_lens:
+            cu.append(cu[-1] + ln)
+        ints = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+        self.seg_lens, self.num_segments, self.num_tokens = list(seg_lens), len(seg_lens), cu[-1]
+        self.cu_seqlens, self.state_slots, self.state_phase = ints(cu), ints(slots), ints(phases)
+        self.scratch = {}
+
+
+def _matrix_memory_float64(rows, gates, b_gates, norm_w, H, dk, dv, cap, eps, floor, state, seg_lens, slots, phases):
+    """The recurrence written out, float64 on the host: outputs [N, H dv] and the states behind every segment."""
+    rows, gates, b_gates, norm_w, state = (t.double().cpu() for t in (rows, gates, b_gates, norm_w, state))
+    n = rows.shape[0]
+    q = rows[:, : H * dk].reshape(n, H, dk) * dk ** -0.5
+    k = rows[:, H * dk: 2 * H * dk].reshape(n, H, dk)
+    v = rows[:, 2 * H * dk: 2 * H * dk + H * dv].reshape(n, H, dv)
+    z = cap * torch.tanh((gates + b_gates) / cap)
+    li, lf = z[:, :H], torch.nn.functional.logsigmoid(z[:, H:])
+    out = torch.zeros(n, H, dv, dtype=torch.float64)
+    new_state = state.clone()
+    t = 0
+    for ln, slot, ph in zip(seg_lens, slots, phases):
+        st = state[slot, ph]
+        C, nn_, m = st[:, : dk * dv].reshape(H, dk, dv).clone(), st[:, dk * dv: dk * dv + dk].clone(), st[:, -1].clone()
+        for _ in range(ln):
+            m2 = torch.maximum(lf[t] + m, li[t])
+            keep, take = torch.exp(lf[t] + m - m2), torch.exp(li[t] - m2)
+            C = keep[:, None, None] * C + take[:, None, None] * k[t][:, :, None] * v[t][:, None, :]
+            nn_ = keep[:, None] * nn_ + take[:, None] * k[t]
+            m = m2
+            den = torch.maximum((nn_ * q[t]).sum(-1).abs(), torch.exp(-m)) + floor
+            out[t] = torch.einsum("hkv,hk->hv", C, q[t]) / den[:, None]
+            t += 1
+        new_state[slot, 1 - ph] = torch.cat([C.reshape(H, dk * dv), nn_, m[:, None]], dim=1)
+    o = out / torch.sqrt(out.pow(2).mean(-1, keepdim=True) + eps)
+    o = o.reshape(n, H * dv) * norm_w * torch.sigmoid(rows[:, 2 * H * dk + H * dv:])
+    return o, new_state
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("H,dk,dv", [(2, 16, 16), (3, 24, 40), (1, 10, 6), (4, 64, 128), (2, 128, 64), (2, 7, 70), (1, 100, 130)])
+@pytest.mark.parametrize("gates_at", ["middle", "forgetting", "keeping"])
+def test_matrix_memory_in_chunks_equals_token_by_token(ops, ref, monkeypatch, dt, H, dk, dv, gates_at):
+    """Segments that end before, at and behind a chunk's edge, single tokens beside them, states that are not zero
+    and whose running maximum is far from the gates, slots in any order and either half: the chunked kernels
+    against the plain recurrence, outputs and new states; and the same step without chunks."""
+    seg_lens = [200, 1, 64, 7, 65, 1, 63, 128, 9]
+    ctx = _Segments(seg_lens, slots=[3, 0, 8, 5, 1, 7, 2, 4, 6], phases=[0, 1, 1, 0, 0, 1, 0, 1, 0])
+    n = ctx.num_tokens
+    g = torch.Generator().manual_seed(H * 100 + dk)
+    rows = (torch.randn(n, 2 * H * dk + 2 * H * dv, generator=g)).to(dt).to(DEV)
+    shift = {"middle": 0.0, "forgetting": -6.0, "keeping": 9.0}[gates_at]
+    gates = (torch.randn(n, 2 * H, generator=g) * 3.0).to(DEV)
+    gates[:, H:] += shift
+    b_gates = torch.randn(2 * H, generator=g).to(DEV)
+    norm_w = (torch.rand(H * dv, generator=g) + 0.5).to(DEV)
+    state = torch.randn(9, 2, H, dk * dv + dk + 1, generator=g).to(DEV)
+    state[:, :, :, -1] = torch.randn(9, 2, H, generator=g).to(DEV) * 8.0  # running maxima
+    st_got, st_scan = state.clone(), state.clone()
+    slots, phases = ctx.state_slots.tolist(), ctx.state_phase.tolist()
+    want, st_ref = _matrix_memory_float64(rows, gates, b_gates, norm_w, H, dk, dv, 12.0, 1e-5, 1e-6, state, seg_lens,
+                                          slots, phases)
+    calls = []
+    inner = ops._call
+    monkeypatch.setattr(ops, "_call", lambda name, *a: (calls.append(name), inner(name, *a))[1])
+    got = ops.mlstm(rows, gates.clone(), b_gates, norm_w, H, dk, dv, 12.0, 1e-5, 1e-6, st_got, ctx)
+    assert calls == ["jle_mlstm_chunked"]
+    monkeypatch.setattr(type(ops), "MLSTM_CHUNKS_FROM", 10 ** 9)
+    scan = ops.mlstm(rows, gates.clone(), b_gates, norm_w, H, dk, dv, 12.0, 1e-5, 1e-6, st_scan, ctx)
+    assert calls[-1] == "jle_mlstm"
+    # (under strong forgetting n . q can be a small difference of large terms: the token-by-token kernel's float32
+    # sums then lose a digit more than the chunks' sums on the matrix instruction)
+    for name, other, tol32 in (("chunks", got, 1e-4), ("token by token", scan, 1e-3)):
+        assert torch.isfinite(other).all(), name
+        err = float((other.double().cpu() - want).abs().max())
+        assert err < (tol32 if dt == torch.float32 else 2e-2), (name, err)
+    for name, st in (("chunks", st_got), ("token by token", st_scan)):
+        for slot, ph in zip(slots, phases):  # the halves that the step wrote
+            a, b = st[slot, 1 - ph].double().cpu(), st_ref[slot, 1 - ph]
+            assert float(((a - b).abs() / b.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)).max()) < 1e-5, (name, slot)
+            assert torch.equal(st[slot, ph], state[slot, ph]), "the half that the step reads stays as it was"
+
+
 def _distance_table(hq, length, seed):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(hq, length, generator=g) * 1.5).to(DEV)
