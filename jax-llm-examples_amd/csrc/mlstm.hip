@@ -302,6 +302,23 @@ __device__ __forceinline__ void chunk_gates(const float* __restrict__ gates, int
 template <typename T>
 __device__ __forceinline__ void stage_rows(const T* __restrict__ rows, int width, int t0, int n, int first, int cols,
                                            int padded, int stride, float mul, float* dst) {
+  constexpr int V = sizeof(T) == 2 ? 8 : 4;  // elements of a 16-byte load
+  if (cols % V == 0 && first % V == 0 && width % V == 0) {
+    const int per_row = padded / V;  // (padded is a multiple of 16, stride of 4)
+    for (int idx = threadIdx.x; idx < kChunk * per_row; idx += blockDim.x) {
+      const int s = idx / per_row, c = (idx - s * per_row) * V;
+      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+      if (s < n && c < cols) {
+        const T* src = rows + (size_t)(t0 + s) * width + first + c;
+        lo = load_v4<T>(src);
+        if (V == 8) hi = load_v4<T>(src + 4);
+      }
+      *reinterpret_cast<f32x4*>(dst + s * stride + c) = f32x4{lo[0] * mul, lo[1] * mul, lo[2] * mul, lo[3] * mul};
+      if (V == 8)
+        *reinterpret_cast<f32x4*>(dst + s * stride + c + 4) = f32x4{hi[0] * mul, hi[1] * mul, hi[2] * mul, hi[3] * mul};
+    }
+    return;
+  }
   for (int idx = threadIdx.x; idx < kChunk * padded; idx += blockDim.x) {
     const int s = idx / padded, c = idx - s * padded;
     float v = 0.f;
@@ -449,9 +466,18 @@ __global__ __launch_bounds__(256) void mlstm_chunk_out_kernel(const T* __restric
   stage_rows<T>(rows, width, t0, n, H * dk + h * dk, dk, dkp, KS, 1.0f, sK);
   stage_rows<T>(rows, width, t0, n, 2 * H * dk + h * dv + c0, min(kSlice, dv - c0), kSlice, VS, 1.0f, sV);
   const float* C0 = ws_C + ((size_t)chunk * H + h) * dk * dv;
-  for (int idx = threadIdx.x; idx < dkp * kSlice; idx += 256) {
-    const int k = idx / kSlice, c = idx - k * kSlice;
-    sC[k * VS + c] = (k < dk && c0 + c < dv) ? C0[(size_t)k * dv + c0 + c] : 0.f;
+  if (dv % 4 == 0) {  // (four columns a load: they are there together or not at all)
+    for (int idx = threadIdx.x; idx < dkp * (kSlice / 4); idx += 256) {
+      const int k = idx / (kSlice / 4), c = (idx - k * (kSlice / 4)) * 4;
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (k < dk && c0 + c < dv) v = *reinterpret_cast<const f32x4*>(C0 + (size_t)k * dv + c0 + c);
+      *reinterpret_cast<f32x4*>(sC + k * VS + c) = v;
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < dkp * kSlice; idx += 256) {
+      const int k = idx / kSlice, c = idx - k * kSlice;
+      sC[k * VS + c] = (k < dk && c0 + c < dv) ? C0[(size_t)k * dv + c0 + c] : 0.f;
+    }
   }
   for (int k = threadIdx.x; k < dkp; k += 256) s_n[k] = k < dk ? ws_n[((size_t)chunk * H + h) * dk + k] : 0.f;
   __syncthreads();
