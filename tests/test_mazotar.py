@@ -68,7 +68,7 @@ def test_distance_buckets():
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("streams,width", [(1, 54), (2, 64), (4, 1000), (3, 2304), (7, 40)])
+@pytest.mark.parametrize("streams,width", [(1, 54), (2, 64), (4, 1000), (3, 2304), (7, 40), (9, 72), (16, 128), (5, 4608)])
 def test_residual_streams_alone(device, streams, width):
     """The update of all streams at once from the old ones, the weighted sum and its norm, for a plain branch output;
     then the plain sum of the streams (what the model's end norms)."""
