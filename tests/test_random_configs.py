@@ -3,7 +3,7 @@ widths and vocabularies that are no power of two, one to seventeen experts with 
 between them, chunks that are no multiple of the page size, three page sizes, with and without frequency scaling,
 q/k norm and temperature.  Each runs a mixed trace (portions beside single tokens, pages used again) in float32 and
 bfloat16 against the plain implementation: the kernels take every size the configuration allows.  The same for the
-Tiradra design (``draw_tiradra``)."""
+Tiradra design (``draw_tiradra``) and the Mazotar design (``draw_mazotar``)."""
 import random
 
 import pytest
@@ -146,4 +146,91 @@ def test_random_tiradra_configuration(tmp_path, seed, dtype):
         assert torch.isfinite(got[rid]).all(), f"{top}: {rid}: non-finite logits"
         err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
         bad = (err > {"float32": 3e-5, "bfloat16": 5e-2}[dtype]).nonzero().squeeze(-1).tolist()
+        assert not bad, f"{top}, page size {page_size}: {rid}: first wrong position {bad[0]}, error {err[bad[0]]:.3g}"
+
+
+# ---------------------------------------------------------------------------------------------- the Mazotar design
+def draw_mazotar(seed: int):
+    """Every size and option of the design at random: no, one or up to nine streams, head sizes that do and do not fit
+    the matrix-core attention kernels, values smaller and larger than keys, distance tables of 4 to 70 rows that end
+    before and beyond the prompts, layers that borrow keys and values from any earlier attention layer, matrix
+    memories with keys of 5 to 128 and values of 3 to 130 elements, dense and routed feed-forwards or none."""
+    rng = random.Random(2000 + seed)
+    width = rng.choice([40, 54, 64, 72, 96, 128, 136, 200, 256])
+
+    def mlp():
+        kind = rng.choice(["none", "dense", "moe", "moe"])
+        if kind == "none":
+            return None
+        if kind == "dense":
+            return {"kind": "dense", "ff": rng.choice([24, 40, 64, 128, 320])}
+        experts = rng.choice([1, 2, 3, 5, 8, 17])
+        m = {"kind": "moe", "router": {"experts": experts, "top": rng.randint(1, min(experts, 3))},
+             "expert": {"ff": rng.choice([16, 24, 64, 128])}}
+        if rng.random() < 0.6:
+            m["shared"] = {"ff": rng.choice([16, 40, 128])}
+        return m
+
+    layers, lenders = [], []
+    for i in range(rng.randint(1, 6)):
+        if rng.random() < 0.4:
+            m = {"heads": rng.choice([1, 2, 3, 5]), "dim": rng.choice([5, 8, 16, 24, 64, 100, 128]),
+                 "vdim": rng.choice([3, 8, 16, 40, 64, 128, 130]), "gate_cap": rng.choice([4.0, 15.0, 30.0])}
+            layers.append({"type": "mlstm", "mixer": m, "mlp": mlp()})
+            continue
+        if lenders and rng.random() < 0.35:
+            j = rng.choice(lenders)
+            m = dict(layers[j]["mixer"], kv_from=j, scale=rng.choice([0.1, 0.3]))
+        else:
+            kv = rng.choice([1, 2, 3, 4])
+            dim = rng.choice([6, 8, 16, 20, 32, 48, 64, 96, 128])
+            m = {"heads": kv * rng.choice([1, 2, 3, 8]), "kv_heads": kv, "dim": dim,
+                 "vdim": rng.choice([dim, dim, 4, 24, 32, 64, 128]), "scale": rng.choice([dim ** -0.5, 0.2, 0.6])}
+            lenders.append(i)
+        rows = rng.choice([4, 6, 9, 16, 32, 70])
+        m["bias_rows"] = rows
+        m["bias_max"] = rng.choice([d for d in (3, 5, 9, 20, 64, 128, 1000) if d > rows // 2])
+        m.pop("q_temp", None)
+        if rng.random() < 0.6:
+            m["q_temp"] = {"coef": rng.choice([0.1, 0.5]), "every": rng.choice([3, 16, 64, 8192])}
+        layers.append({"type": "attention", "mixer": m, "mlp": mlp()})
+    top = {"architecture": "Mazotar", "vocab": rng.choice([97, 257, 300, 512, 1001]), "width": width,
+           "norm": {"eps": rng.choice([1e-5, 1e-6, 1e-3])}, "layers": layers}
+    if rng.random() < 0.8:
+        top["streams"] = rng.choice([1, 2, 3, 4, 4, 9])
+    if rng.random() < 0.7:
+        top["embedding"] = {"scale": rng.choice([0.5, 1.0, 3.0])}
+    lengths = [rng.choice([1, 2, 7, 8, 17, 33, 64, 65, 97, 130, 200]) for _ in range(rng.randint(2, 5))]
+    return top, rng.choice([16, 16, 32, 64]), lengths
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_random_mazotar_configuration(tmp_path, seed, dtype):
+    from plain_mazotar import PlainMazotar
+
+    top, page_size, lengths = draw_mazotar(seed)
+    arch = get_architecture(top["architecture"])
+    folder = write_random_model(arch, arch.parse_config(top), str(tmp_path / "m"), seed,
+                                torch.float32 if dtype == "float32" else torch.bfloat16)
+    reqs = traces.random_requests(top["vocab"], lengths, seed=seed)
+    steps = traces.mixed(reqs, seed=seed)
+    runner = make_runner(folder, dtype, traces.max_live_tokens(steps), "cuda:0", page_size=page_size, poison=True,
+                         max_requests=4)
+    routes = {}
+    if dtype == "bfloat16":  # (a router's close call may fall the other way: the plain model is told the choices)
+        got, routes = traces.run_trace(runner, steps, record_routing=True)
+    else:
+        got = traces.run_trace(runner, steps)
+    runner.cache.check()
+    assert runner.cache.num_live() == 0
+    plain = PlainMazotar.from_dir(folder)
+    for rid, toks in reqs.items():
+        choices = {li: ids.long() for li, ids in routes[rid].items()} if rid in routes else None
+        ref = plain.forward(toks, choices=choices).float()
+        assert torch.isfinite(got[rid]).all(), f"{top}: {rid}: non-finite logits"
+        err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
+        # (a sequence's first tokens leave a matrix memory as sign(q . k) v / rms while exp(-m) is small: where q . k is
+        # near zero that is steep, and two such layers behind each other double the rounding's reach)
+        bad = (err > {"float32": 1e-4, "bfloat16": 1e-1}[dtype]).nonzero().squeeze(-1).tolist()
         assert not bad, f"{top}, page size {page_size}: {rid}: first wrong position {bad[0]}, error {err[bad[0]]:.3g}"
