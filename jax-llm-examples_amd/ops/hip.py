@@ -1169,6 +1169,7 @@ class HipOps:
         return self.paged_attention(q, kv_cache, block_table, positions, token_segment, retention, scale, meta)
 
     PREFILL_TILE = 32  # tokens per prefill work item (the kernels take 16 or 32)
+    BIASED_TILE = 16  # the same for the kernel with a distance bias and sinks
     GENERIC_SPLIT_BELOW = 2048  # the float32-arithmetic attention: fewer (token, head) pairs than this share their keys
     DECODE_MIN_SPLIT = 128  # decode attention: keys per work item (wavefront) at least ...
     DECODE_FIT_SPLIT = 1024  # ... and at most
@@ -1194,7 +1195,8 @@ class HipOps:
             return min(whole, (int(retention[1]) - 1) // split + 2)
         return whole
 
-    def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1, group_size=1, decode_bucket=None):
+    def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1, group_size=1, decode_bucket=None,
+                       tile=None):
         """Work lists of the MFMA attention kernels for one step and one retention rule: the rows that are
         single decode tokens (and into how many keys their work is split), tiles of up to 32 consecutive
         tokens of longer segments and, with ``group_size`` > 1 query heads per kv head, the packing of the
@@ -1205,6 +1207,7 @@ class HipOps:
         from ..parts.base import first_needed_position
 
         dec, tiles, spans, seg_tiles = [], [], [], []
+        tile = tile or self.PREFILL_TILE
         o = 0
         for i, n in enumerate(seg_lens):
             if n == 1:
@@ -1213,8 +1216,8 @@ class HipOps:
                     spans.append((first_needed_position(retention, seg_starts[i]), seg_starts[i]))
             else:
                 first = len(tiles) // 2
-                for t in range(0, n, self.PREFILL_TILE):
-                    tiles += [o + t, min(self.PREFILL_TILE, n - t)]
+                for t in range(0, n, tile):
+                    tiles += [o + t, min(tile, n - t)]
                 seg_tiles.append((first, len(tiles) // 2 - first, seg_starts[i] + n - 1))
             o += n
         split, max_splits = self.DECODE_MAX_SPLIT, 1
@@ -1238,7 +1241,7 @@ class HipOps:
             split = best[1]
             max_splits = max(ranges_of(split))
         groups = []
-        if tiles and group_size > 1 and self.PREFILL_TILE == 32:
+        if tiles and group_size > 1 and tile == 32:
             # consecutive (tile, head) items of one segment, `waves` per block; blocks with the most keys first
             waves = int(self._query("jle_attention_group_waves"))
             keyed = []
@@ -1247,7 +1250,7 @@ class HipOps:
                 for lo in range(0, items, waves):
                     n_items = min(waves, items - lo)
                     last_tile = first + (lo + n_items - 1) // group_size
-                    end = last_pos - (first + count - 1 - last_tile) * self.PREFILL_TILE  # about where its keys end
+                    end = last_pos - (first + count - 1 - last_tile) * tile  # about where its keys end
                     keyed.append((-end, len(keyed), [first + lo // group_size, lo % group_size, n_items, 0]))
             keyed.sort()
             groups = [v for _, _, quad in keyed for v in quad]
@@ -1305,18 +1308,19 @@ class HipOps:
                 if bias is None:
                     bias = self._zero_bias[(hq, q.device)] = torch.zeros(hq, 1, dtype=torch.float32, device=q.device)
             bias_len = bias.shape[1] if biased else 0
-            key = f"attn_plan_{grouped}"
+            tile = self.BIASED_TILE if biased else self.PREFILL_TILE
+            key = f"attn_plan_{grouped}_{tile}"
             plan = meta.meta.get(key) if meta is not None else None
             if plan is None:
                 seg_lens, seg_starts = self._segments(meta, token_segment, positions)
                 plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk, grouped,
-                                           decode_bucket=meta.decode_bucket if meta is not None else None)
+                                           decode_bucket=meta.decode_bucket if meta is not None else None, tile=tile)
                 if meta is not None:
                     meta.meta[key] = plan
             if plan["num_tiles"]:
                 self._call("jle_attention_prefill", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                            _p(block_table), block_table.shape[1], _p(plan["tiles"]), plan["num_tiles"],
-                           self.PREFILL_TILE, _p(plan["groups"]), plan["num_groups"], mode, param, float(scale), hq,
+                           tile, _p(plan["groups"]), plan["num_groups"], mode, param, float(scale), hq,
                            hk, dh, ps, _p(bias), bias_len, _p(sink))
             if plan["num_dec"]:
                 cols = 16 if hq // hk <= 16 else 32
