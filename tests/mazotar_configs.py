@@ -78,10 +78,10 @@ MAZOTAR = {
 MAZOTAR_FAST = {
     "MF": {
         "seed": 9, "architecture": "Mazotar", "vocab": 1000, "width": 256, "norm": {"eps": 1e-5}, "streams": 4,
-        "embedding": {"scale": 0.5},
+        "embedding": {"scale": 0.8},
         "layers": [
-            _mem(4, 32, 64, 12.0, mlp=_dense(384)),
-            _attn(8, 2, 64, 64, 0.125, 32, 200, temp=(0.3, 128), mlp=_moe(8, 2, 128, shared=128)),
+            _mem(4, 32, 64, 11.0, mlp=_dense(384)),
+            _attn(8, 2, 64, 64, 0.125, 32, 200, temp=(0.25, 96), mlp=_moe(8, 2, 128, shared=128)),
             _attn(4, 4, 128, 96, 0.09, 16, 90, temp=(0.2, 50), mlp=_moe(6, 1, 64, shared=192)),
             _attn(8, 2, 64, 64, 0.1, 64, 1000, kv_from=1, mlp=_dense(256)),
             _mem(2, 128, 128, 6.0, mlp=_moe(4, 1, 128)),

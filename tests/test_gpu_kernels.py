@@ -335,15 +335,15 @@ def test_matrix_memory_in_chunks_equals_token_by_token(ops, ref, monkeypatch, dt
     state[:, :, :, -1] = torch.randn(9, 2, H, generator=g).to(DEV) * 8.0  # running maxima
     st_got, st_scan = state.clone(), state.clone()
     slots, phases = ctx.state_slots.tolist(), ctx.state_phase.tolist()
-    want, st_ref = _matrix_memory_float64(rows, gates, b_gates, norm_w, H, dk, dv, 12.0, 1e-5, 1e-6, state, seg_lens,
+    want, st_ref = _matrix_memory_float64(rows, gates, b_gates, norm_w, H, dk, dv, 9.0, 1e-5, 1e-6, state, seg_lens,
                                           slots, phases)
     calls = []
     inner = ops._call
     monkeypatch.setattr(ops, "_call", lambda name, *a: (calls.append(name), inner(name, *a))[1])
-    got = ops.mlstm(rows, gates.clone(), b_gates, norm_w, H, dk, dv, 12.0, 1e-5, 1e-6, st_got, ctx)
+    got = ops.mlstm(rows, gates.clone(), b_gates, norm_w, H, dk, dv, 9.0, 1e-5, 1e-6, st_got, ctx)
     assert calls == ["jle_mlstm_chunked"]
     monkeypatch.setattr(type(ops), "MLSTM_CHUNKS_FROM", 10 ** 9)
-    scan = ops.mlstm(rows, gates.clone(), b_gates, norm_w, H, dk, dv, 12.0, 1e-5, 1e-6, st_scan, ctx)
+    scan = ops.mlstm(rows, gates.clone(), b_gates, norm_w, H, dk, dv, 9.0, 1e-5, 1e-6, st_scan, ctx)
     assert calls[-1] == "jle_mlstm"
     # (under strong forgetting n . q can be a small difference of large terms: the token-by-token kernel's float32
     # sums then lose a digit more than the chunks' sums on the matrix instruction)
