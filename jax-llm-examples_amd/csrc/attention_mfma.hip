@@ -533,6 +533,7 @@ __global__ __launch_bounds__(WAVES * 64, DH <= 128 ? 2 : 1) void attention_prefi
     col[ct].head = h;
     col[ct].lo = ok ? first_key(ret_mode, ret_param, pos) : 1;
     col[ct].hi = ok ? pos : 0;
+    col[ct].pos = pos;
     const bf16_t* qrow = q + ((size_t)col[ct].token * Hq + h) * DH + g * 8;
 #pragma unroll
     for (int c2 = 0; c2 < KC; ++c2) {
@@ -740,14 +741,18 @@ __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t byte_of
 // half h are those of keys 8 g .. 8 g + 7, and the values are read half by half as one 16-byte piece per element
 // (sv points at the step's value tiles, v_rd is the lane's offset in a tile, tile_bytes the distance between
 // tiles).  halves: 1 if the second half holds nothing for this wavefront.
-template <int DH, int CT, bool MASKED>
+template <int DH, int CT, bool MASKED, bool BIASED = false>
 __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], int halves,
                                                      const unsigned char* sv, uint32_t v_rd, int tile_bytes, int kb,
                                                      const Columns (&col)[CT], int k_lo, int k_hi, float scale_log2,
-                                                     float (&m)[CT], float (&l)[CT], f32x4 (&acc)[CT][DH / 16]) {
+                                                     float (&m)[CT], float (&l)[CT], f32x4 (&acc)[CT][DH / 16],
+                                                     Biasing bias = Biasing{nullptr, 0}, bool far = false,
+                                                     const float* far_b = nullptr) {
   constexpr int DT = DH / 16;
   const int g = (threadIdx.x & 63) >> 4;
+  const float sc = BIASED ? 1.0f : scale_log2;  // (biased scores are scaled where the bias is added)
   bf16x8 pb[CT][2];
+  bf16x8 pb_lo[BIASED ? CT : 1][2];  // (see softmax_and_values)
   float corr[CT];
   bool unchanged = true;
 #pragma unroll
@@ -758,6 +763,15 @@ __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], int hal
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float v = st[ct][tt][i];
+        if (BIASED) {
+          float b = far_b[ct];
+          if (!far) {
+            const int back = col[ct].pos - (kb + 32 * (tt >> 1) + 8 * g + 4 * (tt & 1) + i);
+            b = bias.table[(size_t)col[ct].head * bias.L + min(max(back, 0), bias.L - 1)] * kLog2e;
+          }
+          v = fmaf(v, scale_log2, b);
+          st[ct][tt][i] = v;
+        }
         if (MASKED) {
           const int key = kb + 32 * (tt >> 1) + 8 * g + 4 * (tt & 1) + i;
           const bool ok = key >= col[ct].lo && key <= col[ct].hi;
@@ -767,7 +781,7 @@ __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], int hal
         mx = fmaxf(mx, v);
       }
     mx = column_max(mx);
-    const float m_new = fmaxf(m[ct], mx * scale_log2);  // the scale is positive
+    const float m_new = fmaxf(m[ct], mx * sc);  // the scale is positive
     const float m_use = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
     corr[ct] = __builtin_amdgcn_exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
     unchanged = unchanged && m_new == m[ct];
@@ -777,11 +791,22 @@ __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], int hal
       float p[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        p[j] = __builtin_amdgcn_exp2f(fmaf(st[ct][2 * hf + (j >> 2)][j & 3], scale_log2, -m_use));  // masked: exp2(-inf) = 0
+        p[j] = __builtin_amdgcn_exp2f(fmaf(st[ct][2 * hf + (j >> 2)][j & 3], sc, -m_use));  // masked: exp2(-inf) = 0
         sum += p[j];
       }
       const uint4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
       pb[ct][hf] = __builtin_bit_cast(bf16x8, pk);
+      if (BIASED) {  // what the rounding left out, as a second term
+        float r[8];
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          const uint32_t w = j == 0 ? pk.x : j == 2 ? pk.y : j == 4 ? pk.z : pk.w;
+          r[j] = p[j] - __uint_as_float(w << 16);
+          r[j + 1] = p[j + 1] - __uint_as_float(w & 0xffff0000u);
+        }
+        const uint4 rk = {pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]), pack_bf16(r[4], r[5]), pack_bf16(r[6], r[7])};
+        pb_lo[ct][hf] = __builtin_bit_cast(bf16x8, rk);
+      }
     }
     l[ct] = l[ct] * corr[ct] + sum;
     m[ct] = m_new;
@@ -829,17 +854,22 @@ __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], int hal
     for (int dt = 0; dt < DT; ++dt) {
       const bf16x8 a = __builtin_bit_cast(bf16x8, vraw[dt]);
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CT; ++ct) {
+        if (BIASED) acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb_lo[ct][hf], acc[ct][dt], 0, 0, 0);
         acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct][hf], acc[ct][dt], 0, 0, 0);
+      }
     }
   }
 }
 
+// BIASED: a distance bias on every score and, with `sink`, one more term in every head's denominator (two blocks a
+// compute unit all the same: 86 us against 99 with one, at 2,048 tokens, 16 heads on 8 kv heads).
+template <bool BIASED>
 __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ tiles, const int* __restrict__ groups, int ret_mode, int ret_param,
-    float scale_log2, int Hq, int Hkv, int ps) {
+    float scale_log2, int Hq, int Hkv, int ps, Biasing bias, const float* __restrict__ sink) {
   constexpr int DH = 128, CT = 2, KC = DH / 32, DT = DH / 16;
   constexpr int NB = 2;
   constexpr int TILE = 16 * DH * 2;  // bytes of a key tile, and of a value tile
@@ -884,6 +914,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
     col[ct].head = h;
     col[ct].lo = ok ? first_key(ret_mode, ret_param, pos) : 1;
     col[ct].hi = ok ? pos : 0;
+    col[ct].pos = pos;
     const bf16_t* qrow = q + ((size_t)col[ct].token * Hq + h) * DH + g * 8;
 #pragma unroll
     for (int c2 = 0; c2 < KC; ++c2) {
@@ -898,6 +929,13 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
   }
   int all_lo, all_hi;
   common_range<CT>(col, all_lo, all_hi);
+  float far_b[CT];         // with a distance bias: the table's last entry, and the last key that is that far behind
+  int far_until = INT_MIN;  // every live column of the wavefront (its columns' positions ascend: the first is the least)
+  if (BIASED) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) far_b[ct] = bias.table[(size_t)h * bias.L + bias.L - 1] * kLog2e;
+    far_until = p_first - (bias.L - 1);
+  }
 
   // What this wavefront fetches of a step: key tile `wave` and value tile `wave`, four kilobytes each.  Byte offsets
   // from the tile's first key / first value column:
@@ -996,7 +1034,15 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
             for (int ct = 0; ct < CT; ++ct)
               st[ct][2 * hf + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[t][c], qb[ct][c], st[ct][2 * hf + t], 0, 0, 0);
       }
-      if (kb >= all_lo && kb + 63 <= all_hi)  // the same for the whole wavefront
+      if (BIASED) {
+        const bool far = kb + 63 <= far_until;
+        if (kb >= all_lo && kb + 63 <= all_hi)
+          softmax64_and_values<DH, CT, false, true>(st, 2, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m,
+                                                    l, acc, bias, far, far_b);
+        else
+          softmax64_and_values<DH, CT, true, true>(st, halves, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi,
+                                                   scale_log2, m, l, acc, bias, far, far_b);
+      } else if (kb >= all_lo && kb + 63 <= all_hi)  // the same for the whole wavefront
         softmax64_and_values<DH, CT, false>(st, 2, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
       else  // (keys outside a column's range, those of tiles that were not asked for among them, count for nothing)
         softmax64_and_values<DH, CT, true>(st, halves, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
@@ -1011,7 +1057,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     if (ct * 16 + c16 >= nt) continue;
-    const float sum = column_sum(l[ct]);
+    float sum = column_sum(l[ct]);
+    if (BIASED && sink != nullptr) sum += exp2f(sink[h] * kLog2e - m[ct]);
     const float inv = bad ? __builtin_nanf("") : (sum > 0.f ? 1.0f / sum : 0.f);
     bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
 #pragma unroll
@@ -1446,7 +1493,7 @@ JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, cons
   if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps)) return JLE_BAD_ARG;
   // bias: [Hq][bias_len] (with a sink and no bias: a table of zeros); the kernels that share keys take neither
   if ((bias == nullptr) != (bias_len == 0) || (sink != nullptr && bias == nullptr)) return JLE_BAD_ARG;
-  if (bias != nullptr && groups != nullptr) return JLE_BAD_ARG;
+  if (bias != nullptr && groups != nullptr && dh != 128) return JLE_BAD_ARG;  // (of those, the kernel for 128 alone)
   const Biasing bs = {bias, bias_len};
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
   const long long items = (long long)num_tiles * Hq;
@@ -1466,9 +1513,14 @@ JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, cons
       case 64: PICK_S(64); break;
       case 96: PICK_S(96); break;
       case 128:  // (the kernel whose loads go straight into shared memory)
-        hipLaunchKernelGGL(attention_prefill_lds_kernel, gs, dim3(kGroupWaves * 64), 0, s, (const bf16_t*)q,
-                           (const bf16_t*)kv, (bf16_t*)out, positions, token_segment, block_table, table_width, tiles,
-                           groups, ret_mode, ret_param, sl, Hq, Hkv, ps);
+        if (bias != nullptr)
+          hipLaunchKernelGGL(attention_prefill_lds_kernel<true>, gs, dim3(kGroupWaves * 64), 0, s, (const bf16_t*)q,
+                             (const bf16_t*)kv, (bf16_t*)out, positions, token_segment, block_table, table_width, tiles,
+                             groups, ret_mode, ret_param, sl, Hq, Hkv, ps, bs, sink);
+        else
+          hipLaunchKernelGGL(attention_prefill_lds_kernel<false>, gs, dim3(kGroupWaves * 64), 0, s, (const bf16_t*)q,
+                             (const bf16_t*)kv, (bf16_t*)out, positions, token_segment, block_table, table_width, tiles,
+                             groups, ret_mode, ret_param, sl, Hq, Hkv, ps, bs, sink);
         break;
       case 256: PICK_S(256); break;
     }

@@ -1301,14 +1301,15 @@ class HipOps:
             self._chk(sink, torch.float32, (hq,), "sinks")
         if (q.dtype == torch.bfloat16 and hq // hk <= 32
                 and self._query("jle_attention_mfma_supported", dh, hq, hk, ps)):
-            # (with a bias or sinks: every (tile, head) a wavefront of its own, no keys shared between wavefronts)
-            grouped = 1 if biased else hq // hk
+            # (with a bias or sinks the kernel for heads of 128 alone shares keys between wavefronts; at other sizes
+            # every (tile, head) is a wavefront of its own, in tiles of 16 tokens)
+            grouped = hq // hk if (not biased or dh == 128) else 1
             if biased and bias is None:
                 bias = self._zero_bias.get((hq, q.device))
                 if bias is None:
                     bias = self._zero_bias[(hq, q.device)] = torch.zeros(hq, 1, dtype=torch.float32, device=q.device)
             bias_len = bias.shape[1] if biased else 0
-            tile = self.BIASED_TILE if biased else self.PREFILL_TILE
+            tile = self.BIASED_TILE if biased and grouped == 1 else self.PREFILL_TILE
             key = f"attn_plan_{grouped}_{tile}"
             plan = meta.meta.get(key) if meta is not None else None
             if plan is None:

@@ -388,6 +388,21 @@ def test_attention_with_distance_bias_and_sinks(ops, ref, monkeypatch, dt, hq, h
         _assert_close_to_scale(got, want, dt)
 
 
+@pytest.mark.parametrize("hq,hk,ps", [(10, 2, 16), (16, 8, 16), (6, 3, 32), (9, 3, 48), (4, 2, 64)])
+@pytest.mark.parametrize("length", [1, 70, 400, 1300])
+def test_biased_attention_of_long_portions_at_head_size_128(ops, ref, hq, hk, ps, length):
+    """The kernel that shares a step's keys between the wavefronts of a block, with a distance table and sinks:
+    portions of hundreds of tokens behind hundreds of cached ones, tables that end inside a step of 64 keys, before
+    the portion and beyond every context."""
+    dt = torch.bfloat16
+    q, kv, bt, pos, seg = _attention_case(hq, hk, 128, ps, dt, [(0, 333), (190, 130), (517, 1), (64, 64), (1000, 35)], seed=3)
+    bias = _distance_table(hq, length, seed=length + 1)
+    sink = torch.linspace(-4.0, 6.0, hq).to(DEV)
+    got = ops.paged_attention(q, kv, bt, pos, seg, ("all",), 128 ** -0.5, bias=bias, sink=sink)
+    want = ref.paged_attention(q, kv, bt, pos, seg, ("all",), 128 ** -0.5, bias=bias, sink=sink)
+    _assert_close_to_scale(got, want, dt)
+
+
 @pytest.mark.parametrize("dh", [64, 128])
 @pytest.mark.parametrize("back", [0, 1, 30, 31, 32, 63, 64, 65, 200])
 def test_a_distance_table_entry_that_stands_out_picks_its_key(ops, ref, dh, back):
