@@ -83,6 +83,7 @@ class CacheView:
     group: Optional[int] = None
     pages: Optional[dict] = None  # further per-token tensors of this run, by name: [pages, page_size, *shape]
     run_state: Optional[dict] = None  # the arrangement's per-request state of this run, by name: [slots, 2, *shape]
+    states: Optional[dict] = None  # the mixer's further per-request state (``CacheNeed.states``), by name: [slots, *shape]
 
 
 def group_key(need: CacheNeed):
@@ -213,6 +214,12 @@ class CacheManager:
                 self.state[cid] = torch.zeros(
                     (max_requests, *need.state_shape), dtype=need.state_dtype or torch.float32, device=self.device
                 )
+        self.named_state: dict[int, dict[str, torch.Tensor]] = {}
+        for cid in sorted(needs):
+            if needs[cid].states:
+                self.named_state[cid] = {
+                    name: torch.zeros((max_requests, *shape), dtype=dt or dtype, device=self.device)
+                    for name, shape, dt in needs[cid].states}
         # State that an arrangement keeps per run of the order (``run_states``: place in the order -> {name: (shape,
         # dtype)}), in two halves: a step reads the half that the request's last committed step wrote and writes
         # the other (``state_phase``), so a step that is run again before its commit - a recorded step is run
@@ -241,7 +248,7 @@ class CacheManager:
         slot = self.slots.alloc()
         for t in self.state.values():
             t[slot].zero_()
-        for named in self.run_state.values():
+        for named in list(self.run_state.values()) + list(self.named_state.values()):
             for t in named.values():
                 t[slot].zero_()
         self._lives += 1

@@ -92,3 +92,4 @@ def _ensure_builtin() -> None:
     from ..parts import rovidra as _rovidra  # noqa: F401
     from ..parts import tiradra as _tiradra  # noqa: F401
     from ..parts import mazotar as _mazotar  # noqa: F401
+    from ..parts import sudilorn as _sudilorn  # noqa: F401

@@ -131,6 +131,12 @@ class ReferenceOps:
             return t if delta.weight is None else t * delta.weight.float()
         if hasattr(delta, "a"):  # a BranchSum
             return delta.a.float() if delta.b is None else delta.a.float() + delta.b.float()
+        if hasattr(delta, "terms"):  # a ScaledSum: vector * sum_i factor_i * term_i
+            total = None
+            for t, f in delta.terms:
+                piece = self.materialize(t).float() * f
+                total = piece if total is None else total + piece
+            return total if delta.vector is None else total * delta.vector.float()
         return delta
 
     def add_norm_pair(self, x, delta, injected, weight_a, weight_b, eps: float, out_dtype, second: bool = False,
@@ -288,6 +294,120 @@ class ReferenceOps:
             kv_cache[page, 0, :, off] = pad(k).to(kv_cache.dtype)
             values_t(kv_cache)[page, :, :, off] = pad(v).to(kv_cache.dtype)
         return pad(q).to(dt).contiguous()
+
+    def conv_rows(self, proj, bias, conv_w, taps: int, state, ctx, activation=None):
+        """``u = proj + bias`` rounded to the run dtype; ``y[t] = sum_j conv_w[j] * u[t - taps + 1 + j]`` per channel
+        (``conv_w``: float32 ``[taps, channels]``; without taps ``y = u``), the rows before a segment's start from
+        the request's state (``state[slot, phase]``: ``[taps - 1, channels]``, oldest first; zeros before the
+        sequence's start), whose other half gets the last ``taps - 1`` rows of ``u``; ``activation = "silu"``:
+        ``y * sigmoid(y)``; ``[N, channels]`` rounded to the run dtype."""
+        dt = ctx.dtype
+        u = proj.float() if bias is None else (proj.float() + bias.float())
+        u = u.to(dt).float()
+        y = u
+        if taps:
+            y = torch.zeros_like(u)
+            cu = ctx.cu_seqlens.tolist()
+            slots, phase = ctx.state_slots.tolist(), ctx.state_phase.tolist()
+            w = conv_w.float()
+            for s in range(len(cu) - 1):
+                lo, hi = cu[s], cu[s + 1]
+                rows = u[lo:hi]
+                if taps > 1:
+                    rows = torch.cat([state[slots[s], phase[s]].float(), rows], dim=0)
+                for j in range(taps):
+                    y[lo:hi] += w[j] * rows[j: j + hi - lo]
+                if taps > 1:
+                    state[slots[s], 1 - phase[s]] = rows[rows.shape[0] - (taps - 1):].to(state.dtype)
+        if activation == "silu":
+            y = y * torch.sigmoid(y)
+        elif activation is not None:
+            raise ValueError(f"unknown activation {activation!r}")
+        return y.to(dt)
+
+    def heads_prepare(self, rows, q_heads: int, k_heads: int, v_heads: int, head_dim: int, value_dim: int,
+                      page_dim: int, prep, positions, kv_cache, slot_mapping):
+        """``rows``: ``[N, q_heads dk + k_heads dk + v_heads dv]`` = q | k | v.  q and k per head: ``prep``'s RMS
+        norm (weights of ``dk`` elements or none, before or after the rotation) and rotation (adjacent or half-split
+        pairs of the leading elements, sines and cosines times the magnitude); k and v written into their pages
+        (if ``kv_cache`` is given: ``k_heads`` heads of ``page_dim`` elements, zeros behind the real ones; value head
+        ``j`` goes to the ``k_heads / v_heads`` key heads ``j * share .. (j + 1) * share - 1``).  Returns q ``[N,
+        q_heads, page_dim]`` in the run dtype."""
+        n = rows.shape[0]
+        dt = rows.dtype
+        dk, dv, D = head_dim, value_dim, page_dim
+        r = rows.float()
+        q = r[:, : q_heads * dk].reshape(n, q_heads, dk)
+        k = r[:, q_heads * dk: (q_heads + k_heads) * dk].reshape(n, k_heads, dk)
+        v = r[:, (q_heads + k_heads) * dk:].reshape(n, v_heads, dv)
+
+        def norm(x, w):
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + prep.norm_eps)
+            return x if w is None else x * w.float()
+
+        if prep.norm_eps is not None and prep.norm_first:
+            q, k = norm(q, prep.norm_weight_q), norm(k, prep.norm_weight_k)
+        q, k = self._turn(q, positions, prep.rotation), self._turn(k, positions, prep.rotation)
+        if prep.norm_eps is not None and not prep.norm_first:
+            q, k = norm(q, prep.norm_weight_q), norm(k, prep.norm_weight_k)
+        pad = lambda t: torch.nn.functional.pad(t, (0, D - t.shape[-1]))
+        if kv_cache is not None:
+            ps = kv_cache.shape[3]
+            page, off = (slot_mapping // ps).long(), (slot_mapping % ps).long()
+            kv_cache[page, 0, :, off] = pad(k).to(kv_cache.dtype)
+            values_t(kv_cache)[page, :, :, off] = pad(v).repeat_interleave(k_heads // v_heads, dim=1).to(kv_cache.dtype)
+        return pad(q).to(dt).contiguous()
+
+    def diff_combine(self, o, lam: float, out_scale: float, eps: float, gate, num_heads: int, num_kv_heads: int,
+                     page_dim: int, value_dim: int):
+        """``o``: ``[N, 2 H page_dim]``, the outputs of the two score maps in the order ``[kv head][map][query head
+        of the group]``.  Per head ``d = a1 - lam * a2`` over its ``value_dim`` real elements, divided by its root
+        mean square (``eps``), times ``out_scale`` and, with ``gate`` (``[N, H value_dim]``), times its sigmoid;
+        ``[N, H value_dim]`` in the heads' own order, run dtype."""
+        n = o.shape[0]
+        H, G = num_heads, num_kv_heads
+        a = o.float().reshape(n, G, 2, H // G, page_dim)[..., :value_dim]
+        d = (a[:, :, 0] - lam * a[:, :, 1]).reshape(n, H, value_dim)
+        d = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * out_scale
+        d = d.reshape(n, H * value_dim)
+        if gate is not None:
+            d = d * torch.sigmoid(gate.float())
+        return d.to(o.dtype)
+
+    def gated_delta(self, rows, gates, a_log, dt_bias, norm_weight, out_gate, num_heads: int, num_kv_heads: int,
+                    head_dim: int, value_dim: int, eps: float, floor: float, state, ctx):
+        """``rows``: ``[N, 2 G dk + H dv]`` = q | k | v behind convolution and activation, run dtype; ``gates``:
+        float32 ``[N, 2 H]`` = the write strengths' and the decays' pre-activations.  Per kv head q and k become unit
+        vectors (``x / sqrt(sum(x^2) + floor)``), q times ``dk^(-1/2)``; ``beta = sigmoid(.)``, ``g = exp(-exp(a_log)
+        softplus(. + dt_bias))``; per head, token by token from the request's memory (``state[slot, phase]``: ``[H,
+        dk, dv]``; the new one goes to ``state[slot, 1 - phase]``): ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
+        o = S^T q``.  Then ``o`` divided by its root mean square per head (``eps``), times ``norm_weight`` (``[dv]``),
+        times ``silu(out_gate)``.  ``[N, H dv]`` in the run dtype."""
+        n = rows.shape[0]
+        H, G, dk, dv = num_heads, num_kv_heads, head_dim, value_dim
+        r = rows.float()
+        q = r[:, : G * dk].reshape(n, G, dk)
+        k = r[:, G * dk: 2 * G * dk].reshape(n, G, dk)
+        v = r[:, 2 * G * dk:].reshape(n, H, dv)
+        q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + floor) * (dk ** -0.5)
+        k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + floor)
+        q, k = q.repeat_interleave(H // G, dim=1), k.repeat_interleave(H // G, dim=1)
+        beta = torch.sigmoid(gates[:, :H].float())
+        decay = torch.exp(-torch.exp(a_log.float()) * torch.nn.functional.softplus(gates[:, H:].float() + dt_bias.float()))
+        out = torch.empty(n, H, dv, dtype=torch.float32, device=rows.device)
+        cu = ctx.cu_seqlens.tolist()
+        slots, phase = ctx.state_slots.tolist(), ctx.state_phase.tolist()
+        for s in range(len(cu) - 1):
+            S = state[slots[s], phase[s]].float().clone()
+            for t in range(cu[s], cu[s + 1]):
+                S = decay[t][:, None, None] * S
+                u = beta[t][:, None] * (v[t] - torch.einsum("hkv,hk->hv", S, k[t]))
+                S = S + k[t][:, :, None] * u[:, None, :]
+                out[t] = torch.einsum("hkv,hk->hv", S, q[t])
+            state[slots[s], 1 - phase[s]] = S.to(state.dtype)
+        o = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        g = out_gate.float()
+        return (o.reshape(n, H * dv) * (g * torch.sigmoid(g))).to(rows.dtype)
 
     def batched_linear(self, a, w, tokens_first: bool = False):
         """``out[b] = a[b] @ w[b]`` for ``a [B, N, K]`` and ``w [B, K, M]`` (views with any strides);
@@ -483,11 +603,16 @@ class ReferenceOps:
         hk, ps = kv_cache.shape[2], kv_cache.shape[3]
         g = hq // hk
         out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
+        keep = 0
+        if retention[0] == "window_keep":  # the window's keys and the sequence's first `keep` tokens
+            keep, retention = int(retention[2]), ("window", retention[1])
         starts = retention_start(retention, positions)
         for i in range(n):
             p = int(positions[i])
             s = int(starts[i])
             kpos = torch.arange(s, p + 1, device=q.device)
+            if keep and s > 0:
+                kpos = torch.cat([torch.arange(0, min(keep, s), device=q.device), kpos])
             pages = block_table[int(token_segment[i])][(kpos // ps).long()].long()
             if bool((pages < 0).any()):
                 raise RuntimeError(f"token {i} at position {p} reads a page that was given back")
@@ -546,6 +671,45 @@ class ReferenceOps:
                 h32, w = shared_gate
                 shared = (shared.float() * torch.sigmoid(h32.float() @ w.float().reshape(-1, 1))).to(shared.dtype)
             out += shared.float()
+        return out
+
+    def moe_choose(self, h32, router, correction, top_k: int, groups=None, keep_groups=None, group_terms: int = 2):
+        """Router logits ``z`` in float32, scores ``s = sigmoid(z)``, choice scores ``c = s + correction``
+        (``correction``: float32 ``[E]`` or ``None``).  With ``groups``: the experts form that many equal groups of
+        neighbours, a group's score is the sum of its ``group_terms`` largest ``c``, the ``keep_groups`` best groups
+        (lowest index first among equals) stay and the others' experts cannot be chosen.  The ``top_k`` largest ``c``
+        among those that can, lowest index first among equals.  Returns ``(ids int32 [N, top_k], their s float32,
+        None)`` (the third: the grouping by expert that a kernel set may make in the same call)."""
+        z = h32.float() @ router.float().t()
+        s = torch.sigmoid(z)
+        c = s if correction is None else s + correction.float()
+        n, e = c.shape
+        if groups is not None:
+            per = e // groups
+            gs = torch.sort(c.view(n, groups, per), dim=-1, descending=True).values[..., :group_terms].sum(-1)
+            kept = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep_groups]
+            allowed = torch.zeros(n, groups, dtype=torch.bool, device=c.device)
+            allowed.scatter_(1, kept, True)
+            c = c.masked_fill(~allowed.repeat_interleave(per, dim=1), float("-inf"))
+        ids = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :top_k]
+        return ids.to(torch.int32), torch.gather(s, 1, ids), None
+
+    def moe_experts_scored(self, h, expert_ids, weights, w_up, w_down, activation: str = "relu2", tiled: bool = False,
+                           grouping=None):
+        """``sum_j weights[j] * W_down[e_j] act(W_up[e_j] h)`` per token, float32 result; ``w_up`` ``[E, F, D]``,
+        ``w_down`` ``[E, D, F]``; ``act = relu2``: the square of relu.  Activations between the two products and
+        every expert's weighted output are rounded to the run dtype, as the kernels store them."""
+        assert not tiled, "the plain ops read row-major weights"
+        if activation != "relu2":
+            raise ValueError(f"unknown activation {activation!r}")
+        n, d = h.shape
+        out = torch.zeros(n, d, dtype=torch.float32, device=h.device)
+        hf = h.float()
+        for j in range(expert_ids.shape[1]):
+            for e in torch.unique(expert_ids[:, j]).tolist():
+                rows = (expert_ids[:, j] == e).nonzero().squeeze(-1)
+                act = (torch.relu(hf[rows] @ w_up[e].float().t()) ** 2).to(h.dtype).float()
+                out[rows] += ((act @ w_down[e].float().t()) * weights[rows, j: j + 1].float()).to(h.dtype).float()
         return out
 
     # ------------------------------------------------------------------ sampling

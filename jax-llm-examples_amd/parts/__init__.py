@@ -1,4 +1,5 @@
-from . import attention, embedding, feed_forward, latent_attention, mlstm, norm, position  # noqa: F401  (register the built-in parts)
+from . import (attention, embedding, feed_forward, gated_delta, latent_attention, mlstm, norm, position,  # noqa: F401
+               side_by_side)  # noqa: F401  (register the built-in parts)
 from .base import (CacheNeed, Embedding, FeedForward, Mixer, Norm, OutputHead, ParamSpec, Part, PositionEncoding,
                    build_embedding, build_feed_forward, build_head, register_embedding, register_head,
                    build_mixer, build_norm, build_position, first_needed_position, register_feed_forward, register_retention,

@@ -18,7 +18,16 @@ logarithm of the distance up to ``max_distance``, where the last row begins), ``
 whose exponential is one more term of the softmax's denominator) and ``own_kv = False`` (the layer projects no keys
 and values: its run reads the cache that another run writes).  With any of these the rows go through
 ``qkv_span_prepare`` (norms over the projections, query scale, pages with heads filled up with zeros) and the
-attention kernels that take a bias table and sinks.  Formulas:
+attention kernels that take a bias table and sinks.  A third family, off for Llama 4 too: ``score_maps``
+(``differential``: every head has two score maps, each a softmax of its own with queries and keys of its own over the
+same values; with ``lam = exp(lq1 . lk1) - exp(lq2 . lk2) + diff`` from four learned vectors the head's output is
+``a1 - lam a2``, divided by its root mean square and multiplied by ``1 - diff``; q and k rows lie head by head as
+``[map 1, map 2]``), ``output_gate`` (the heads side by side times ``sigmoid(W_g h)`` before the output projection),
+a weighted q/k norm before the rotation together with a convolution, half-split pairs with a stretch, and the
+retention rule ``window_keep`` (a window plus the sequence's first tokens).  With any of these the projected rows go
+through ``conv_rows`` (bias, convolution, state), ``heads_prepare`` (norm, rotation, pages with filled-up heads; a
+value head written once per score map, so that the attention kernels see ``maps * kv_heads`` key/value heads, the
+queries re-ordered at load so that those of a key head lie together) and, for two maps, ``diff_combine``.  Formulas:
 ``llama4/llama4_jax/model.py:891-955`` (projections, rotation, q/k norm, order of
 the cache write) and ``model.py:745-794`` (scores times ``softmax_scale``, causal
 mask, float32 softmax, values).
@@ -86,21 +95,37 @@ class Attention(Mixer):
         self.biased = bool(spec.get("bias", False))
         self.conv_taps = int(spec.get("conv_taps") or 0)
         rot = self.position.rotation()
+        maps = spec.get("score_maps")
+        if maps is not None and maps.kind != "differential":
+            raise ValueError(f"unknown score_maps kind {maps.kind!r}")
+        self.maps = 1 if maps is None else 2
+        self.diff = None if maps is None else float(maps.diff)
+        self.head_norm_eps = None if maps is None else float(maps.eps)
+        self.output_gate = bool(spec.get("output_gate", False))
+        # the path through conv_rows and heads_prepare (see the module's text)
+        self.general = (self.maps > 1 or self.output_gate or self.retention[0] == "window_keep"
+                        or ((self.conv_taps > 0 or self.biased or self.value_dim != self.head_dim)
+                            and (self.qk_norm_weighted or self.qk_norm_first
+                                 or (rot is not None and rot.pairing != "adjacent"))))
+        self.lam = None
         if self.spanned:
             if self.qk_norm_span != "projection" or not self.qk_norm_weighted or self.qk_norm_first:
                 raise ValueError("distance_bias, sink and own_kv=False come with a weighted q/k norm over the projection")
             if rot is not None or self.biased or self.conv_taps:
                 raise ValueError("the attention mixer's path with a q/k norm over the projection has no rotation, no "
                                  "projection bias and no convolution")
+        if self.general and (self.spanned or self.query_scale is not None or self.qk_norm_span != "head"):
+            raise ValueError("score maps, an output gate, the window_keep rule and a weighted norm with a convolution "
+                             "come without a norm over the projection, a distance table, sinks and a query scale")
         # the path through the convolution kernel, which also rotates, norms, fills up and writes the pages
-        self.convolved = not self.spanned and (self.conv_taps > 0 or self.value_dim != self.head_dim or self.biased
+        self.convolved = not self.spanned and not self.general and (self.conv_taps > 0 or self.value_dim != self.head_dim or self.biased
                                                or (rot is not None and rot.magnitude != 1.0))
         if self.convolved and (self.qk_norm_weighted or self.qk_norm_first or self.query_scale is not None):
             raise ValueError("the attention mixer's convolution path norms q and k without weights after the rotation "
                              "and has no query scale")
         # the head size of the pages
         self.page_dim = self.head_dim if not self.convolved else -(-max(self.head_dim, self.value_dim) // 8) * 8
-        if self.spanned:  # (from 32 on a multiple of 32: the sizes the matrix-core attention kernels take)
+        if self.spanned or self.general:  # (from 32 on a multiple of 32: the sizes the matrix-core attention kernels take)
             widest = max(self.head_dim, self.value_dim)
             self.page_dim = -(-widest // 32) * 32 if widest >= 32 else -(-widest // 8) * 8
         self.state_dtype = None
@@ -123,8 +148,13 @@ class Attention(Mixer):
             extra["bqkv"] = ParamSpec((channels,), policy="float32", init=("normal", 0.3))
         if self.conv_taps:
             extra["conv"] = ParamSpec((channels, self.conv_taps), policy="float32", init=("normal", 0.6))
+        if self.output_gate:
+            extra["wg"] = ParamSpec((hq * dv, d), init=("normal", d ** -0.5))
+        if self.maps > 1:
+            for name in ("lam_q1", "lam_k1", "lam_q2", "lam_k2"):
+                extra[name] = ParamSpec((dh,), policy="float32", init=("normal", 0.3))
         return {
-            # rows: q heads, then k heads, then v heads; each [out, in]
+            # rows: q heads (head by head, a head's score maps one after the other), then k heads, then v heads
             "wqkv": ParamSpec((channels, d)),
             "wo": ParamSpec((d, hq * dv)),
             **extra,
@@ -137,7 +167,7 @@ class Attention(Mixer):
     def channels(self) -> int:
         if not self.own_kv:  # (queries only)
             return self.num_heads * self.head_dim
-        return (self.num_heads + self.num_kv_heads) * self.head_dim + self.num_kv_heads * self.value_dim
+        return (self.num_heads + self.num_kv_heads) * self.maps * self.head_dim + self.num_kv_heads * self.value_dim
 
     def distance_table(self) -> torch.Tensor:
         """The learned table told per head and distance, float32 ``[heads, max_distance + 1]``: column ``n`` is what a
@@ -151,6 +181,12 @@ class Attention(Mixer):
         self.state_dtype = dtype
 
     def cache_need(self) -> CacheNeed:
+        if self.general:  # (the attention kernels see a key/value head per score map)
+            kv = (self.num_kv_heads * self.maps, self.page_dim)
+            if self.conv_taps > 1:
+                return CacheNeed(kv=kv, retention=self.retention, state_shape=(2, self.conv_taps - 1, self.channels),
+                                 state_dtype=self.state_dtype)
+            return CacheNeed(kv=kv, retention=self.retention)
         if self.conv_taps > 1:  # [half, tap, channel]: the last taps - 1 projected rows, as the projection left them
             return CacheNeed(kv=(self.num_kv_heads, self.page_dim), retention=self.retention,
                              state_shape=(2, self.conv_taps - 1, self.channels), state_dtype=self.state_dtype)
@@ -173,8 +209,23 @@ class Attention(Mixer):
             self.bias_run = self.params["bqkv"].to(self.params["wqkv"].dtype)
         # a tap's weights of all channels side by side, as the kernels read them
         self.conv_by_tap = self.params["conv"].t().contiguous() if self.conv_taps else None
+        if self.maps > 1 and self.lam is None:
+            # the queries of a key head (a kv head's map) next to each other: [kv head][map][query head of the group]
+            P = self.params
+            self.lam = float(torch.exp((P["lam_q1"].double() * P["lam_k1"].double()).sum())
+                             - torch.exp((P["lam_q2"].double() * P["lam_k2"].double()).sum()) + self.diff)
+            r, dh = self.num_heads // self.num_kv_heads, self.head_dim
+            order = [((g * r + j) * self.maps + mp) * dh + e for g in range(self.num_kv_heads)
+                     for mp in range(self.maps) for j in range(r) for e in range(dh)]
+            nq = len(order)
+            idx = torch.tensor(order, device=P["wqkv"].device)
+            for name in ("wqkv", "bqkv", "conv"):
+                if name in P:
+                    P[name][:nq] = P[name][:nq][idx]
+            self.bias_run = None if not self.biased else P["bqkv"].to(P["wqkv"].dtype)
+            self.conv_by_tap = P["conv"].t().contiguous() if self.conv_taps else None
         self.wo_padded = None
-        if self.page_dim != self.value_dim:  # the attention's output has page_dim elements a head: zeros' columns
+        if self.page_dim != self.value_dim and self.maps == 1:  # the attention's output has page_dim elements a head: zeros' columns
             wo = self.params["wo"]
             padded = torch.zeros(wo.shape[0], self.num_heads, self.page_dim, dtype=wo.dtype, device=wo.device)
             padded[:, :, : self.value_dim] = wo.view(wo.shape[0], self.num_heads, self.value_dim)
@@ -187,6 +238,25 @@ class Attention(Mixer):
 
     def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
         ops = ctx.ops
+        if self.general:
+            mp = self.maps
+            proj, bias = ops.linear_bias(h, self.params["wqkv"], self.params.get("bqkv"), self.bias_run)
+            gate = ops.linear(h, self.params["wg"]) if self.output_gate else None
+            rows = ops.conv_rows(proj, bias, self.conv_by_tap, self.conv_taps, cache.state, ctx)
+            q = ops.heads_prepare(rows, self.num_heads * mp, self.num_kv_heads * mp, self.num_kv_heads, self.head_dim,
+                                  self.value_dim, self.page_dim, self.prep, ctx.positions,
+                                  cache.kv if cache.writes else None, cache.slot_mapping)
+            o = ops.paged_attention(q, cache.kv, cache.block_table, ctx.positions, ctx.token_segment, self.retention,
+                                    self.softmax_scale, cache.attn_meta)
+            if mp > 1:
+                o = ops.diff_combine(o, self.lam, 1.0 - self.diff, self.head_norm_eps, gate, self.num_heads,
+                                     self.num_kv_heads, self.page_dim, self.value_dim)
+                return ops.linear(o, self.params["wo"])
+            if gate is not None:
+                if self.page_dim != self.value_dim:
+                    raise ValueError("an output gate on heads that are filled up with zeros is not provided for")
+                o = ops.sigmoid_mul(o, gate)
+            return ops.linear(o, self.params["wo"] if self.wo_padded is None else self.wo_padded)
         if self.spanned:
             if cache.writes != self.own_kv:
                 raise ValueError("a run writes its cache if and only if its layer projects keys and values")

@@ -83,7 +83,8 @@ class CacheNeed:
     ``paged``: further per-token tensors in pages (see below).
     ``retention``: which earlier tokens a query at position ``p`` may still read:
     ``("all",)``; ``("chunk", C)``: those with ``pos >= (p // C) * C``;
-    ``("window", W)``: those with ``pos > p - W``; or any rule registered with
+    ``("window", W)``: those with ``pos > p - W``; ``("window_keep", W, K)``: those and the first ``K`` positions of
+    the sequence; or any rule registered with
     :func:`register_retention`.  Pages that hold only tokens no later query can read are given back.
     ``state_shape``/``state_dtype``: fixed-size state per request (``None`` if the mixer has none).
     """
@@ -99,6 +100,11 @@ class CacheNeed:
     # (``CacheView.pages[name]``).  ``kv`` is the layout the attention kernels read (keys ``[page_size,
     # head_dim]`` and values transposed in one tensor).
     paged: tuple = ()
+    # Further fixed-size state per request, by name: a tuple of ``(name, shape, dtype)``; each becomes a tensor
+    # ``[slots, *shape]``, cleared when a request is admitted, that the mixer finds in ``CacheView.states[name]``
+    # (a mixer that keeps a recurrent memory in float32 beside a convolution's last rows in the run dtype; a mixer
+    # made of several, each with state of its own).
+    states: tuple = ()
 
 
 @dataclasses.dataclass(frozen=True)
@@ -137,6 +143,10 @@ register_retention("chunk", lambda rule, next_pos: (next_pos // int(rule[1])) * 
                    lambda rule, step: int(rule[1]) + step)
 register_retention("window", lambda rule, next_pos: max(0, next_pos - int(rule[1]) + 1),
                    lambda rule, step: int(rule[1]) + step)
+# ("window_keep", W, K): the window's keys and, for ever, the sequence's first K tokens
+register_retention("window_keep", lambda rule, next_pos: max(0, next_pos - int(rule[1]) + 1),
+                   # (the prefix's pages and the window's are rounded to pages apart: room for a page of up to 256 tokens)
+                   lambda rule, step: int(rule[1]) + int(rule[2]) + step + 256, lambda rule: int(rule[2]))
 
 
 def first_needed_position(retention: tuple, next_pos: int) -> int:

@@ -12,7 +12,7 @@ import torch
 
 from ..config.specs import LayerSpec
 from .base import ParamSpec, Part, build_feed_forward, build_mixer, build_norm
-from .residual import BranchSum, GatedBranch
+from .residual import BranchSum, GatedBranch, ScaledSum
 
 _ARRANGEMENTS = {}
 
@@ -33,8 +33,31 @@ def build_block(spec: LayerSpec):
     return cls(spec)
 
 
+class ChannelScale(Part):
+    """A learned factor per channel on a branch's output (float32); the kernel that adds the branch to the residual
+    multiplies."""
+
+    graph_safe = True
+
+    def __init__(self, hidden: int) -> None:
+        super().__init__()
+        self.hidden = int(hidden)
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.hidden,), policy="float32", init=("uniform", 0.5, 1.5))}
+
+    def flops_per_token(self) -> float:
+        return 0.0
+
+
 @register_arrangement("pre_norm")
 class PreNormBlock:
+    """``x += mixer(norm(x))``, then ``x += feed_forward(norm(x))``.  Options (``LayerSpec.options``), both off for
+    Llama 4: ``branch_mult`` (a number every branch output is multiplied by before the sum) and ``layer_scale`` (with
+    ``hidden_size``: a learned factor per channel on every branch output, :class:`ChannelScale`); with either, what
+    stays pending on the residual is a :class:`~.residual.ScaledSum`.  A mixer may itself return such a sum (two
+    mixers side by side with a weight each)."""
+
     def __init__(self, spec: LayerSpec) -> None:
         self.spec = spec
         self.mixer = build_mixer(spec.mixer)
@@ -43,17 +66,35 @@ class PreNormBlock:
         if spec.feed_forward is not None:
             self.feed_forward = build_feed_forward(spec.feed_forward)
             self.feed_forward_norm = build_norm(spec.feed_forward_norm)
+        opt = spec.options or {}
+        self.branch_mult = float(opt.get("branch_mult", 1.0))
+        self.mixer_scale = self.feed_forward_scale = None
+        if opt.get("layer_scale"):
+            self.mixer_scale = ChannelScale(int(opt["hidden_size"]))
+            if self.feed_forward is not None:
+                self.feed_forward_scale = ChannelScale(int(opt["hidden_size"]))
+        self.scaled = self.branch_mult != 1.0 or self.mixer_scale is not None
 
     def parts(self):
         out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm}
+        if self.mixer_scale is not None:
+            out["mixer_scale"] = self.mixer_scale
         if self.feed_forward is not None:
             out.update(feed_forward=self.feed_forward, feed_forward_norm=self.feed_forward_norm)
+            if self.feed_forward_scale is not None:
+                out["feed_forward_scale"] = self.feed_forward_scale
         return out
+
+    def _branch(self, y, scale):
+        if not self.scaled:
+            return y
+        return ScaledSum.of(y, self.branch_mult, None if scale is None else scale.params["weight"])
 
     def forward(self, residual, ctx, cache) -> None:
         want32 = bool(getattr(self.mixer, "wants_float32_input", False))
         h, h32 = self.mixer_norm.forward(residual, ctx, want32=want32)
-        residual.add(self.mixer.forward(h, ctx, cache, h32) if want32 else self.mixer.forward(h, ctx, cache))
+        y = self.mixer.forward(h, ctx, cache, h32) if want32 else self.mixer.forward(h, ctx, cache)
+        residual.add(self._branch(y, self.mixer_scale))
         ff = self.feed_forward
         if ff is None:
             return
@@ -61,7 +102,7 @@ class PreNormBlock:
             h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=ff.wants_float32_input, defer=True)
         else:
             h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=ff.wants_float32_input)
-        residual.add(ff.forward(h, h32, ctx))
+        residual.add(self._branch(ff.forward(h, h32, ctx), self.feed_forward_scale))
 
 
 @register_arrangement("parallel")

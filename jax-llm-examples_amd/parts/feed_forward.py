@@ -121,6 +121,86 @@ class MoESigmoidShared(FeedForward):
                                shared_weights=shared, tiled=self.tiled, grouping=grouping)
 
 
+@register_feed_forward("moe_scored")
+class MoEScored(FeedForward):
+    """Routed experts whose weights are scores, not gates on the input: router logits ``z = W_r h`` in float32,
+    scores ``s = sigmoid(z)``; the ``top_k`` experts with the largest *choice scores* ``s + correction`` (a learned
+    number per expert; option ``correction``) are chosen, lowest index first among equals, and the output is ``sum_e
+    s_e expert_e(h)`` with the scores as they are (no renormalisation).  With ``groups``: the experts form that many
+    equal groups of neighbours, a group's score is the sum of its ``group_score_terms`` largest choice scores, and
+    only experts of the ``keep_groups`` best groups can be chosen.  An expert is ``W_down act(W_up h)`` without
+    biases; ``activation``: ``relu2`` (the square of relu)."""
+
+    wants_float32_input = True
+    graph_safe = True
+
+    def __init__(self, spec) -> None:
+        super().__init__()
+        self.hidden = int(spec.hidden_size)
+        self.num_experts = int(spec.num_experts)
+        self.top_k = int(spec.top_k)
+        self.inter = int(spec.intermediate_size)
+        self.activation = str(spec.get("activation") or "relu2")
+        if self.activation != "relu2":
+            raise ValueError(f"unknown activation {self.activation!r} (relu2)")
+        self.has_correction = bool(spec.get("correction", False))
+        g = spec.get("groups")
+        self.groups = None if g is None else int(g)
+        self.keep_groups = None if g is None else int(spec.keep_groups)
+        self.group_terms = int(spec.get("group_score_terms") or 2)
+        if self.groups is not None and (self.num_experts % self.groups or not 1 <= self.keep_groups <= self.groups
+                                        or self.keep_groups * (self.num_experts // self.groups) < self.top_k):
+            raise ValueError("groups of equal size, 1 <= keep_groups <= groups, and top_k experts within the kept groups")
+        self.tiled = False
+
+    def param_specs(self):
+        e, f, d = self.num_experts, self.inter, self.hidden
+        specs = {
+            "router": ParamSpec((e, d), policy="float32", init=("normal", d ** -0.5)),
+            "w_up": ParamSpec((e, f, d), init=("normal", d ** -0.5)),  # per expert [out, in]
+            "w_down": ParamSpec((e, d, f), init=("normal", f ** -0.5)),
+        }
+        if self.has_correction:
+            specs["correction"] = ParamSpec((e,), policy="float32", init=("normal", 0.3))
+        return specs
+
+    def step_weight_bytes(self, observed=None) -> int:
+        n = self.num_experts if observed is None else int(torch.unique(observed[0]).numel())
+        total = 0
+        for name, t in self.params.items():
+            b = t.numel() * t.element_size()
+            total += b // self.num_experts * n if name in ("w_up", "w_down") else b
+        return total
+
+    def flops_per_token(self) -> float:
+        per = 0
+        for name, t in self.params.items():
+            per += t.numel() // self.num_experts * self.top_k if name in ("w_up", "w_down") else t.numel()
+        return 2.0 * per
+
+    def finalize(self) -> None:
+        from ..ops.layout import can_tile, tile_
+
+        up, dn = self.params["w_up"], self.params["w_down"]
+        if not self.tiled and can_tile(up) and can_tile(dn) and self.inter % 16 == 0:
+            tile_(up)
+            tile_(dn)
+            self.tiled = True
+
+    def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
+        ops = ctx.ops
+        expert_ids, weights, grouping = ops.moe_choose(h32, self.params["router"], self.params.get("correction"),
+                                                       self.top_k, self.groups, self.keep_groups, self.group_terms)
+        tap = getattr(ctx, "tap", None)
+        if tap is not None:  # whoever watches the step sees the choice and may replace it
+            replaced = tap(self, "routing", (expert_ids, weights))
+            if replaced is not None:
+                expert_ids, weights = replaced
+                grouping = None
+        return ops.moe_experts_scored(h, expert_ids, weights, self.params["w_up"], self.params["w_down"],
+                                      activation=self.activation, tiled=self.tiled, grouping=grouping)
+
+
 @register_feed_forward("dense_polynorm")
 class DensePolyNorm(FeedForward):
     """``W_down act(W_up h + b_up) + b_down`` with the polynomial activation

@@ -103,7 +103,8 @@ class DecoderModel:
                 self.loop.enter(residual, embedded, e.enters_pass, ctx)
             gi = cache.group_of.get(e.cache)
             view = CacheView(cache_id=e.cache, writes=e.writes_cache, group=gi, state=cache.state.get(e.cache),
-                             run_state=cache.run_state.get(k))
+                             run_state=cache.run_state.get(k),
+                             states=getattr(cache, "named_state", {}).get(e.cache))
             if gi is not None:
                 g = ctx.groups[gi]
                 view.kv = cache.groups[gi].tensors.get(e.cache)

@@ -94,7 +94,8 @@ def yarn_scaled_frequencies(inv_freq: torch.Tensor, base: float, dims: int, fact
 
 @register_position("rope_yarn")
 class RopeYarn(PositionEncoding):
-    """Rotary embedding over adjacent pairs of the leading ``rotary_dim`` elements (default: all) with frequencies
+    """Rotary embedding over adjacent pairs of the leading ``rotary_dim`` elements (default: all; with the option
+    ``pairing = "half"`` element ``j`` pairs with ``j + rotary_dim / 2`` instead) with frequencies
     ``theta ** (-2 j / rotary_dim)``, optionally stretched (``scaling = (factor, original, fast, slow)``, see
     :func:`yarn_scaled_frequencies`); with a scaling the sines and cosines are also multiplied by
     ``0.1 ln(factor) + 1`` (``Rotation.magnitude``)."""
@@ -112,4 +113,7 @@ class RopeYarn(PositionEncoding):
             factor, original, fast, slow = (float(v) for v in scaling)
             inv = yarn_scaled_frequencies(inv, theta, rd, factor, original, fast, slow)
             magnitude = 0.1 * math.log(factor) + 1.0
-        return Rotation(inv.to(torch.float32), pairing="adjacent", rotary_dim=rd, magnitude=magnitude)
+        pairing = str(self.spec.get("pairing") or "adjacent")
+        if pairing not in ("adjacent", "half"):
+            raise ValueError(f"pairs are 'adjacent' or 'half', not {pairing!r}")
+        return Rotation(inv.to(torch.float32), pairing=pairing, rotary_dim=rd, magnitude=magnitude)

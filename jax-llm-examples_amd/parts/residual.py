@@ -39,6 +39,33 @@ class BranchSum:
         return BranchSum(ops.gather_rows(self.a, idx), None if self.b is None else ops.gather_rows(self.b, idx))
 
 
+class ScaledSum:
+    """A branch output that is not formed yet: ``vector * sum_i factor_i * term_i`` per row, formed in float32 by the
+    kernel that adds it to the residual.  ``terms``: up to two ``(rows, factor)`` pairs, rows ``[N, hidden]`` in the
+    run dtype or float32 (or a sum of expert outputs still in pieces), factors plain numbers; ``vector``: float32
+    ``[hidden]`` or ``None``.  It is what a layer with a multiplier on its branches, a learned scale per channel, or
+    two mixers side by side with a weight each leaves pending."""
+
+    def __init__(self, terms, vector=None) -> None:
+        self.terms = [(t, float(f)) for t, f in terms]
+        if not 1 <= len(self.terms) <= 2:
+            raise ValueError("a scaled sum has one or two terms")
+        self.vector = vector
+        self.shape, self.dtype = self.terms[0][0].shape, self.terms[0][0].dtype
+
+    @classmethod
+    def of(cls, y, factor: float = 1.0, vector=None) -> "ScaledSum":
+        """``vector * factor * y`` where ``y`` is rows or itself a scaled sum (whose own vector must be ``None``)."""
+        if isinstance(y, ScaledSum):
+            if y.vector is not None:
+                raise ValueError("a scaled sum with a vector cannot be scaled by another")
+            return cls([(t, f * factor) for t, f in y.terms], vector)
+        return cls([(y, factor)], vector)
+
+    def rows(self, ops, idx) -> "ScaledSum":
+        return ScaledSum([(ops.gather_rows(t, idx), f) for t, f in self.terms], self.vector)
+
+
 class Residual:
     def __init__(self, x: torch.Tensor) -> None:
         assert x.dtype == torch.float32
