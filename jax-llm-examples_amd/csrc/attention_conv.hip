@@ -37,7 +37,10 @@ struct ConvArgs {
   T* kv_cache;            // [pages, 2, Hkv, ps, D] (values [D][ps]) or null
   float magnitude, norm_eps;  // norm_eps < 0: no norm
   int taps, C, Hq, Hkv, dk, dv, D, ps, rotary_dim;
+  int act;  // (the convolution alone) 1: y * sigmoid(y) before the rounding
 };
+
+__device__ __forceinline__ float conv_act(float y, int act) { return act == 1 ? y / (1.0f + expf(-y)) : y; }
 
 // the projected value of channel c in row `row`, with its bias, as the run dtype holds it
 template <typename PT, typename T>
@@ -174,6 +177,7 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(ConvArgs<PT, T> a, T* __
   float y;
   if (K == 0) {
     y = projected(a, (size_t)n, c);
+    if (a.act) y = Num<T>::round(conv_act(y, a.act));
   } else {
     const int seg = a.token_segment[n];
     const int t = n - a.cu_seqlens[seg];
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(ConvArgs<PT, T> a, T* __
                                     : Num<T>::load(old + (size_t)(K - 1 + t - back) * a.C + c);
       acc = __builtin_fmaf(a.w[(size_t)j * a.C + c], u, acc);
     }
-    y = Num<T>::round(acc);
+    y = Num<T>::round(conv_act(acc, a.act));
   }
   Num<T>::store(y_out + (size_t)n * a.C + c, y);
 }
@@ -273,6 +277,10 @@ __global__ __launch_bounds__(256) void conv_rows_vec_kernel(ConvArgs<PT, T> a, T
     float y[8];
     if (K == 0) {
       projected8(a, (size_t)n, c, bias8, y);
+      if (a.act) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = Num<T>::round(conv_act(y[i], a.act));
+      }
     } else {
       const int seg = a.token_segment[n];
       const int t = n - a.cu_seqlens[seg];
@@ -300,7 +308,7 @@ __global__ __launch_bounds__(256) void conv_rows_vec_kernel(ConvArgs<PT, T> a, T
         for (int i = 0; i < 8; ++i) y[i] = __builtin_fmaf(w8[i], u[i], y[i]);
       }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) y[i] = Num<T>::round(y[i]);
+      for (int i = 0; i < 8; ++i) y[i] = Num<T>::round(conv_act(y[i], a.act));
     }
     Row8<T>::store(y_out + (size_t)n * a.C + c, y);
   }
@@ -375,17 +383,18 @@ JLE_API int jle_conv_qk_prepare(const void* proj, int proj_f32, const float* bia
 }
 
 // The convolution alone: y [N, C] in the run dtype, C channels of any meaning; the state as above.
-JLE_API int jle_conv_rows(const void* proj, int proj_f32, const float* bias, const float* conv_w, int taps,
-                          void* state, const int* token_segment, const int* cu_seqlens, const int* state_slots,
-                          const int* state_phase, void* y_out, int is_bf16, int N, int R, int C, hipStream_t s) {
+static int conv_rows_act(const void* proj, int proj_f32, const float* bias, const float* conv_w, int taps,
+                         void* state, const int* token_segment, const int* cu_seqlens, const int* state_slots,
+                         const int* state_phase, void* y_out, int is_bf16, int N, int R, int C, int act, hipStream_t s) {
   if (N <= 0) return 0;
+  if (act < 0 || act > 1) return JLE_BAD_ARG;
   if (C <= 0 || taps < 0 || R <= 0 || (C + 255) / 256 > 65535 || y_out == nullptr) return JLE_BAD_ARG;
   if ((taps > 0 && conv_w == nullptr) || (taps > 1 && (state == nullptr || state_slots == nullptr || state_phase == nullptr)))
     return JLE_BAD_ARG;
   if (!is_bf16 && !proj_f32) return JLE_BAD_ARG;
 #define JLE_ROWS_ARGS(PT, T)                                                                                        \
   ConvArgs<PT, T> a{(const PT*)proj, bias, conv_w, (T*)state, token_segment, cu_seqlens, state_slots, state_phase, \
-                    nullptr, nullptr, nullptr, nullptr, nullptr, 1.f, -1.f, taps, C, 0, 0, 0, 0, 0, 0, 0}
+                    nullptr, nullptr, nullptr, nullptr, nullptr, 1.f, -1.f, taps, C, 0, 0, 0, 0, 0, 0, 0, act}
   if (!is_bf16) {
     JLE_ROWS_ARGS(float, float);
     return launch_conv_rows(a, y_out, N, R, s);
@@ -397,4 +406,20 @@ JLE_API int jle_conv_rows(const void* proj, int proj_f32, const float* bias, con
   JLE_ROWS_ARGS(bf16_t, bf16_t);
   return launch_conv_rows(a, y_out, N, R, s);
 #undef JLE_ROWS_ARGS
+}
+
+JLE_API int jle_conv_rows(const void* proj, int proj_f32, const float* bias, const float* conv_w, int taps,
+                          void* state, const int* token_segment, const int* cu_seqlens, const int* state_slots,
+                          const int* state_phase, void* y_out, int is_bf16, int N, int R, int C, hipStream_t s) {
+  return conv_rows_act(proj, proj_f32, bias, conv_w, taps, state, token_segment, cu_seqlens, state_slots, state_phase,
+                       y_out, is_bf16, N, R, C, 0, s);
+}
+
+// The same with an activation on the convolution's result (act 1: y * sigmoid(y), float32, before the rounding).
+JLE_API int jle_conv_rows_act(const void* proj, int proj_f32, const float* bias, const float* conv_w, int taps,
+                              void* state, const int* token_segment, const int* cu_seqlens, const int* state_slots,
+                              const int* state_phase, void* y_out, int is_bf16, int N, int R, int C, int act,
+                              hipStream_t s) {
+  return conv_rows_act(proj, proj_f32, bias, conv_w, taps, state, token_segment, cu_seqlens, state_slots, state_phase,
+                       y_out, is_bf16, N, R, C, act, s);
 }

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const int* __restrict__ token_segment, const int* __restrict__ block_table, int table_width, int ret_mode,
     int ret_param, float scale, int N, int Hq, int Hkv, int dh, int ps, int splits, int tiles_per_split,
     float* __restrict__ ws_ml, float* __restrict__ ws_o, const float* __restrict__ bias, int bias_len,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, int keep) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave_index();
   if (item >= N * Hq * splits) return;  // whole wavefront leaves; no block-wide barrier below
@@ -71,9 +71,16 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     t_lo += sp * tiles_per_split * 64;
     t_hi = min(pos, t_lo + tiles_per_split * 64 - 1);
   }
-  for (int t0 = t_lo; t0 <= t_hi; t0 += 64) {
+  // keep > 0: the sequence's first `keep` keys stay visible beside the rule's own; those of them that lie before
+  // the rule's first key are a range of their own, taken (by the first of the wavefronts that share a query) ahead
+  // of the rule's keys
+  const int prefix_end = keep < first ? keep : first;
+  for (int range = (prefix_end > 0 && sp == 0) ? 0 : 1; range < 2; ++range) {
+  const int r_first = range == 0 ? 0 : first, r_last = range == 0 ? prefix_end - 1 : pos;
+  const int r_lo = range == 0 ? 0 : t_lo, r_hi = range == 0 ? r_last : t_hi;
+  for (int t0 = r_lo; t0 <= r_hi; t0 += 64) {
     const int key = t0 + lane;
-    const bool valid = key >= first && key <= pos;
+    const bool valid = key >= r_first && key <= r_last;
     float s = -INFINITY;
     const T* krow = nullptr;
     int voff = 0;
@@ -104,8 +111,8 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     m = m_new;
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] *= corr;
-    const int cnt = (pos - t0 + 1) < 64 ? (pos - t0 + 1) : 64;
-    const int lo = first > t0 ? first - t0 : 0;
+    const int cnt = (r_last - t0 + 1) < 64 ? (r_last - t0 + 1) : 64;
+    const int lo = r_first > t0 ? r_first - t0 : 0;
     if (ps % 16 == 0) {
       // pages hold whole groups of 16 keys: a lane reads the 16 values of its head elements in one piece
       // (values lie [head_dim][page_size]) and adds them up with the probabilities broadcast by shuffle
@@ -154,6 +161,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
         }
       }
     }
+  }
   }
   bad = __any(bad);
   if (splits > 1) {
@@ -248,8 +256,9 @@ static int launch_generic(const void* q, const void* kv, void* out, const int* p
                           const int* block_table, int table_width, int ret_mode, int ret_param, float scale,
                           int is_bf16, int N, int Hq, int Hkv, int dh, int ps, int splits, int tiles_per_split,
                           float* ws_ml, float* ws_o, const float* bias, int bias_len, const float* sink,
-                          hipStream_t s) {
+                          hipStream_t s, int keep = 0) {
   if (N <= 0) return 0;
+  if (keep < 0) return JLE_BAD_ARG;
   if (bias != nullptr && bias_len < 1) return JLE_BAD_ARG;
   if (dh % 8 || dh > 256 || Hkv <= 0 || Hq % Hkv || ps <= 0) return JLE_BAD_ARG;
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
@@ -261,7 +270,7 @@ static int launch_generic(const void* q, const void* kv, void* out, const int* p
   if (is_bf16) {
     hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,
                        (bf16_t*)out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale,
-                       N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink);
+                       N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink, keep);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(paged_attention_generic_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, N * Hq,
@@ -269,7 +278,7 @@ static int launch_generic(const void* q, const void* kv, void* out, const int* p
   } else {
     hipLaunchKernelGGL(paged_attention_generic_kernel<float>, g, b, 0, s, (const float*)q, (const float*)kv,
                        (float*)out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale, N,
-                       Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink);
+                       Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink, keep);
     JLE_LAUNCH_CHECK();
     if (splits > 1)
       hipLaunchKernelGGL(paged_attention_generic_merge_kernel<float>, gm, b, 0, s, ws_ml, ws_o, (float*)out, N * Hq, dh,
@@ -295,6 +304,15 @@ JLE_API int jle_paged_attention_biased(const void* q, const void* kv, void* out,
                                        const float* bias, int bias_len, const float* sink, hipStream_t s) {
   return launch_generic(q, kv, out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale,
                         is_bf16, N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, bias, bias_len, sink, s);
+}
+
+// The same under a rule that also keeps the sequence's first `keep` keys visible (a window with kept first tokens).
+JLE_API int jle_paged_attention_kept(const void* q, const void* kv, void* out, const int* positions,
+                                     const int* token_segment, const int* block_table, int table_width, int ret_mode,
+                                     int ret_param, int keep, float scale, int is_bf16, int N, int Hq, int Hkv, int dh,
+                                     int ps, int splits, int tiles_per_split, float* ws_ml, float* ws_o, hipStream_t s) {
+  return launch_generic(q, kv, out, positions, token_segment, block_table, table_width, ret_mode, ret_param, scale,
+                        is_bf16, N, Hq, Hkv, dh, ps, splits, tiles_per_split, ws_ml, ws_o, nullptr, 0, nullptr, s, keep);
 }
 
 // The merge alone, for kernels that leave their key ranges' results in the same layout (attention_f32.hip).

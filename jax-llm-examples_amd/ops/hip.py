@@ -13,7 +13,8 @@ import torch
 
 from . import build as _build
 
-_RET_MODES = {"all": 0, "chunk": 1, "window": 2}  # the rules under which the attention kernels here read keys
+# the rules under which the attention kernels here read keys ("window_keep": the general kernel alone)
+_RET_MODES = {"all": 0, "chunk": 1, "window": 2, "window_keep": 2}
 
 
 def _ret_mode(retention) -> int:
@@ -87,6 +88,17 @@ _SIGNATURES = {
                           _i, _i, _f, _f, _f, _vp],
     "jle_span_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_row_gate": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
+    "jle_scaled_add_norm": [_vp, _vp, _i, _f, _vp, _i, _f, _vp, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
+    "jle_heads_prepare": [_vp, _vp, _vp, _vp, _i, _i, _f, _f, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i,
+                          _vp],
+    "jle_diff_combine": [_vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gated_delta": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
+                        _i, _i, _i, _f, _f, _vp],
+    "jle_moe_choose": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_relu2": [_vp, _vp, _i, _ll, _vp],
+    "jle_conv_rows_act": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "jle_paged_attention_kept": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
+                                 _vp, _vp],
     "jle_paged_attention_biased": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                                    _vp, _vp, _i, _vp, _vp],
 }
@@ -624,7 +636,31 @@ class HipOps:
                    _p(sink))
         return out
 
+    def scaled_add_norm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False, norm: bool = True):
+        """``x += vector * sum_i factor_i * term_i`` in place for a :class:`~..parts.residual.ScaledSum` (terms in the
+        run dtype or float32; a sum of expert outputs still in pieces is formed first), then (``norm``) ``h = x /
+        sqrt(mean(x^2) + eps) * weight`` in the run dtype and, if wanted, float32; one launch."""
+        n, d = x.shape
+        self._chk(x, torch.float32, (n, d), "residual")
+        terms = [(self.materialize(t), f) for t, f in delta.terms]
+        for t, _ in terms:
+            self._chk(t, None, (n, d), "branch output")
+        kind = lambda t: 1 if t.dtype == torch.bfloat16 else 2 if t.dtype == torch.float32 else self._is_bf16(t)
+        (a, fa), (b, fb) = terms[0], (terms[1] if len(terms) > 1 else (None, 0.0))
+        if delta.vector is not None:
+            self._chk(delta.vector, torch.float32, (d,), "channel scale")
+        if weight is not None:
+            self._chk(weight, torch.float32, (d,), "norm weight")
+        h = torch.empty(n, d, dtype=out_dtype, device=x.device) if norm else None
+        h32 = torch.empty(n, d, dtype=torch.float32, device=x.device) if norm and want32 else None
+        self._call("jle_scaled_add_norm", _p(x), _p(a), kind(a), float(fa), _p(b), 0 if b is None else kind(b),
+                   float(fb), _p(delta.vector), _p(weight), float(eps), _p(h),
+                   1 if out_dtype == torch.bfloat16 else 0, _p(h32), n, d)
+        return h, h32
+
     def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):
+        if hasattr(delta, "terms"):  # a sum with factors: the kernel that knows it
+            return self.scaled_add_norm(x, delta, weight, eps, out_dtype, want32)
         if hasattr(delta, "a"):  # the sum of two parallel branches: the kernel that knows it
             h, _ = self.add_norm_pair(x, delta, None, weight, None, eps, out_dtype)
             return h, (h.float() if want32 else None)
@@ -669,6 +705,9 @@ class HipOps:
         return out
 
     def add_residual(self, x, delta) -> None:
+        if hasattr(delta, "terms"):
+            self.scaled_add_norm(x, delta, None, 0.0, torch.float32, norm=False)
+            return
         if hasattr(delta, "a"):
             self.add_norm_pair(x, delta, None, None, None, 0.0, delta.dtype, norm=False)
             return
@@ -768,7 +807,7 @@ class HipOps:
                                  page_dim, prep, ctx, kv_cache if writes else None, slot_mapping)
         return self.paged_attention(q, kv_cache, block_table, ctx.positions, ctx.token_segment, retention, scale, meta)
 
-    def conv_rows(self, proj, bias, conv_w, taps: int, state, ctx):
+    def conv_rows(self, proj, bias, conv_w, taps: int, state, ctx, activation=None):
         """``y[t] = sum_j conv_w[j] * u[t - taps + 1 + j]`` (``conv_w``: ``[taps, channels]``) with ``u = proj + bias`` rounded to the run dtype, rows
         before a segment's start from the requests' two-halved state, whose other half gets the segment's last
         ``taps - 1`` rows of ``u``; ``[N, C]`` in the run dtype.  See ``attention_conv.hip``."""
@@ -789,11 +828,92 @@ class HipOps:
                                (ctx.state_phase, "state phases", (ctx.num_segments,))):
             self._chk(t, torch.int32, shape, what)
         y = torch.empty(n, channels, dtype=dt, device=proj.device)
+        if activation is not None:  # (on the convolution's result, float32, before the rounding)
+            if activation != "silu":
+                raise KernelError(f"the convolution kernel knows the activation silu, not {activation!r}")
+            self._call("jle_conv_rows_act", _p(proj), 1 if proj.dtype == torch.float32 else 0, _p(bias),
+                       _p(conv_w) if taps else None, int(taps), _p(state) if taps > 1 else None,
+                       _p(ctx.token_segment), _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(y),
+                       1 if dt == torch.bfloat16 else 0, n, ctx.num_segments, channels, 1)
+            return y
         self._call("jle_conv_rows", _p(proj), 1 if proj.dtype == torch.float32 else 0, _p(bias),
                    _p(conv_w) if taps else None, int(taps), _p(state) if taps > 1 else None, _p(ctx.token_segment),
                    _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(y),
                    1 if dt == torch.bfloat16 else 0, n, ctx.num_segments, channels)
         return y
+
+    def heads_prepare(self, rows, q_heads: int, k_heads: int, v_heads: int, head_dim: int, value_dim: int,
+                      page_dim: int, prep, positions, kv_cache, slot_mapping):
+        """See ``attention_heads.hip``: q and k normed and rotated as ``prep`` says, keys and values into pages with
+        heads of ``page_dim`` elements (a value head once for each of the ``k_heads / v_heads`` key heads that use
+        it).  Returns q ``[N, q_heads, page_dim]``."""
+        n = rows.shape[0]
+        dk, dv, D = head_dim, value_dim, page_dim
+        self._chk(rows, None, (n, (q_heads + k_heads) * dk + v_heads * dv), "projected rows")
+        dt = rows.dtype
+        if prep.query_scale is not None or prep.norm_span != "head":
+            raise KernelError("this preparation kernel has no query scale and norms a head at a time")
+        rot = prep.rotation
+        inv_freq, rd, magnitude, half = None, 0, 1.0, 0
+        if rot is not None:
+            rd = int(rot.rotary_dim) or dk
+            inv_freq, magnitude = self._chk(rot.inv_freq, torch.float32, (rd // 2,), "inv_freq"), float(rot.magnitude)
+            half = 1 if rot.pairing == "half" else 0
+        for w in (prep.norm_weight_q, prep.norm_weight_k):
+            if w is not None:
+                self._chk(w, torch.float32, (dk,), "q/k norm weight")
+        self._chk(positions, torch.int32, (n,), "positions")
+        ps = 1
+        if kv_cache is not None:
+            ps = kv_cache.shape[3]
+            self._chk(kv_cache, dt, (kv_cache.shape[0], 2, k_heads, ps, D), "kv pages")
+            self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
+        q = torch.empty(n, q_heads, D, dtype=dt, device=rows.device)
+        self._call("jle_heads_prepare", _p(rows), _p(positions), _p(slot_mapping) if kv_cache is not None else None,
+                   _p(inv_freq), rd, half, magnitude, -1.0 if prep.norm_eps is None else float(prep.norm_eps),
+                   1 if prep.norm_first else 0, _p(prep.norm_weight_q), _p(prep.norm_weight_k), _p(q), _p(kv_cache),
+                   self._is_bf16(rows), n, q_heads, k_heads, v_heads, dk, dv, D, ps)
+        return q
+
+    def diff_combine(self, o, lam: float, out_scale: float, eps: float, gate, num_heads: int, num_kv_heads: int,
+                     page_dim: int, value_dim: int):
+        """Two score maps' outputs ``[N, 2 H page_dim]`` (``[kv head][map][query head of the group]``) into ``(a1 - lam
+        a2) / rms * out_scale * sigmoid(gate)``, ``[N, H value_dim]`` in the heads' own order."""
+        n = o.shape[0]
+        self._chk(o, None, (n, 2 * num_heads * page_dim), "attention output")
+        if gate is not None:
+            self._chk(gate, o.dtype, (n, num_heads * value_dim), "output gate")
+        out = torch.empty(n, num_heads * value_dim, dtype=o.dtype, device=o.device)
+        self._call("jle_diff_combine", _p(o), _p(gate), _p(out), float(lam), float(out_scale), float(eps),
+                   self._is_bf16(o), n, num_heads, num_kv_heads, page_dim, value_dim)
+        return out
+
+    def gated_delta(self, rows, gates, a_log, dt_bias, norm_weight, out_gate, num_heads: int, num_kv_heads: int,
+                    head_dim: int, value_dim: int, eps: float, floor: float, state, ctx):
+        """See ``gated_delta.hip``: unit vectors, write strengths and decays of the step's tokens, the recurrence
+        from and into the requests' two-halved memory, head norm and output gate.  ``[N, H dv]`` in the run dtype."""
+        n = rows.shape[0]
+        H, G, dk, dv = num_heads, num_kv_heads, head_dim, value_dim
+        self._chk(rows, None, (n, 2 * G * dk + H * dv), "q | k | v rows")
+        self._chk(out_gate, rows.dtype, (n, H * dv), "output gate")
+        self._chk(gates, torch.float32, (n, 2 * H), "gate pre-activations")
+        self._chk(state, torch.float32, (state.shape[0], 2, H, dk, dv), "memory")
+        for t, shape, what in ((a_log, (H,), "a_log"), (dt_bias, (H,), "dt_bias"), (norm_weight, (dv,), "head norm weight")):
+            self._chk(t, torch.float32, shape, what)
+        for t, what, shape in ((ctx.cu_seqlens, "segment bounds", (ctx.num_segments + 1,)),
+                               (ctx.state_slots, "state slots", (ctx.num_segments,)),
+                               (ctx.state_phase, "state phases", (ctx.num_segments,))):
+            self._chk(t, torch.int32, shape, what)
+        dev = rows.device
+        scratch = torch.empty(n * (2 * G * dk + 2 * H + H * dv), dtype=torch.float32, device=dev)
+        qn, kn = scratch[: n * G * dk], scratch[n * G * dk: 2 * n * G * dk]
+        o = 2 * n * G * dk
+        beta, decay, o_raw = scratch[o: o + n * H], scratch[o + n * H: o + 2 * n * H], scratch[o + 2 * n * H:]
+        out = torch.empty(n, H * dv, dtype=rows.dtype, device=dev)
+        self._call("jle_gated_delta", _p(rows), self._is_bf16(rows), _p(gates), _p(a_log), _p(dt_bias), _p(norm_weight),
+                   _p(out_gate), _p(state), _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(qn), _p(kn),
+                   _p(beta), _p(decay), _p(o_raw), _p(out), n, ctx.num_segments, H, G, dk, dv, float(eps), float(floor))
+        return out
 
     def conv_qk_prepare(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
                         value_dim: int, page_dim: int, prep, ctx, kv_cache, slot_mapping):
@@ -1295,6 +1415,9 @@ class HipOps:
         param = int(retention[1]) if len(retention) > 1 else 0
         out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
         biased = bias is not None or sink is not None
+        if retention[0] == "window_keep":
+            return self._attention_kept(q, kv_cache, out, block_table, positions, token_segment, mode, param,
+                                        int(retention[2]), scale, meta, biased)
         if bias is not None:
             self._chk(bias, torch.float32, (hq, bias.shape[1]), "distance bias")
         if sink is not None:
@@ -1406,7 +1529,104 @@ class HipOps:
                    ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o))
         return out
 
+    def _attention_kept(self, q, kv_cache, out, block_table, positions, token_segment, mode: int, param: int,
+                        keep: int, scale: float, meta, biased: bool):
+        """A window whose queries also see the sequence's first ``keep`` keys: the general kernel (float32
+        arithmetic, both dtypes) takes the kept keys that lie before the window as a range of their own."""
+        n, hq, dh = q.shape
+        hk, ps = kv_cache.shape[2], kv_cache.shape[3]
+        if biased:
+            raise KernelError("the attention kernel for kept first tokens takes no distance table and no sinks")
+        if dh % 8 or dh > 256 or hq % hk:
+            raise KernelError(f"attention kernels: head size {dh} (a multiple of 8, at most 256) or {hq} query heads "
+                              f"on {hk} kv heads are not supported")
+        splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
+        waves = n * hq
+        if waves < self.GENERIC_SPLIT_BELOW:  # few tokens with many keys: a query's keys shared between wavefronts
+            if meta is not None and meta.decode_bucket is not None:
+                longest = meta.decode_bucket
+            elif meta is not None:
+                longest = max(s0 + ln for s0, ln in zip(meta.seg_starts, meta.seg_lens))
+            else:
+                longest = int(positions.max()) + 1
+            tiles = -(-min(longest, param + 64) // 64)  # (the window's keys; the kept ones ride with the first range)
+            want = min(tiles, -(-self.GENERIC_SPLIT_BELOW // waves))
+            if want > 1:
+                tiles_per_split = -(-tiles // want)
+                splits = -(-tiles // tiles_per_split)
+                ws_ml = torch.empty(waves * splits * 2, dtype=torch.float32, device=q.device)
+                ws_o = torch.empty(waves * splits * dh, dtype=torch.float32, device=q.device)
+        self._call("jle_paged_attention_kept", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
+                   _p(block_table), block_table.shape[1], mode, param, keep, float(scale), self._is_bf16(q), n, hq, hk,
+                   dh, ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o))
+        return out
+
     # ------------------------------------------------------------------ routed experts
+    def moe_choose(self, h32, router, correction, top_k: int, groups=None, keep_groups=None, group_terms: int = 2):
+        """Router logits in float32 (the router kernel), then the choice by scores with a correction and groups
+        (``moe_choose.hip``) and the grouping of the choices by expert.  Returns ``(ids, weights, grouping)``."""
+        h32 = self._rows(h32, want32=True)
+        n, d = h32.shape
+        e = router.shape[0]
+        self._chk(h32, torch.float32, None, "router input")
+        self._chk(router, torch.float32, (e, d), "router matrix")
+        if correction is not None:
+            self._chk(correction, torch.float32, (e,), "correction")
+        dev = h32.device
+        ids1 = torch.empty(n, 1, dtype=torch.int32, device=dev)
+        gates1 = torch.empty(n, 1, dtype=torch.float32, device=dev)
+        logits = torch.empty(n, e, dtype=torch.float32, device=dev)
+        self._call("jle_moe_route", _p(h32), _p(router), _p(ids1), _p(gates1), _p(logits), n, d, e, 1)
+        ids = torch.empty(n, top_k, dtype=torch.int32, device=dev)
+        weights = torch.empty(n, top_k, dtype=torch.float32, device=dev)
+        self._call("jle_moe_choose", _p(logits), _p(correction), _p(ids), _p(weights), n, e, top_k,
+                   0 if groups is None else int(groups), 0 if groups is None else int(keep_groups), int(group_terms))
+        return ids, weights, self.moe_align(ids, weights, e)
+
+    def relu2(self, x):
+        """``relu(x)^2`` element by element."""
+        self._chk(x, None, None, "rows")
+        y = torch.empty_like(x)
+        self._call("jle_relu2", _p(x), _p(y), self._is_bf16(x), x.numel())
+        return y
+
+    def moe_experts_scored(self, h, expert_ids, weights, w_up, w_down, activation: str = "relu2", tiled: bool = False,
+                           grouping=None):
+        """``sum_j weights[j] * W_down[e_j] relu(W_up[e_j] h)^2``: the choices grouped by expert, the first product
+        plain, the activation a kernel of its own, the weights the second product's row scale (applied to its float32
+        sums); the sum over a token's choices stays in pieces (:class:`ExpertSum`)."""
+        if activation != "relu2":
+            raise KernelError(f"unknown activation {activation!r}")
+        h = self._rows(h)
+        n, d = h.shape
+        e, f, _ = w_up.shape
+        k = expert_ids.shape[1]
+        m = n * k
+        if grouping is None:
+            grouping = self.moe_align(expert_ids.contiguous(), weights.contiguous(), e)
+        offsets, sorted_token, sorted_weight, inv = grouping
+        mfma = h.dtype == torch.bfloat16 and d % 8 == 0 and f % 8 == 0
+
+        def product(x, w, nout, kdim, **kw):
+            if mfma and m <= 2 * self.SKINNY_MAX_ROWS:
+                return self.gemm_skinny(x, w, offsets=offsets, tiled=tiled, **kw)
+            if mfma and tiled and self.stream_supported(nout, kdim, False):
+                return self.gemm_stream(x, w, offsets=offsets, **kw)
+            if mfma:
+                return self.gemm_grouped(x, w, offsets=offsets, tiled=tiled, **kw)
+            if tiled:
+                raise KernelError("weights in the streaming layout need the MFMA product kernels")
+            if (x.dtype == torch.float32 and kdim % 4 == 0 and nout % 4 == 0 and m <= self.F32_SKINNY_ROWS):
+                return self.gemm_f32_skinny(x, w, offsets=offsets, **kw)
+            if (x.dtype == torch.float32 and self.f32_stream_supported(nout, kdim, False) and x.numel() < 2 ** 32
+                    and m * nout < 2 ** 32 and not (x.data_ptr() | w.data_ptr()) % 16):
+                return self.gemm_f32_stream(x, w, offsets=offsets, **kw)
+            return self.gemm(x, w, offsets=offsets, **kw)
+
+        up = product(h, w_up, f, d, a_rows=sorted_token)
+        routed = product(self.relu2(up), w_down, d, f, scale=sorted_weight)
+        return ExpertSum(routed, inv, k, None, n, d)
+
     def moe_route(self, h32, router, top_k: int, want_logits: bool = False, group: bool = False):
         """``group``: also return the grouping of the choices by expert (what ``moe_align`` gives), made in
         the same call; ``moe_experts`` takes it as ``grouping``."""
