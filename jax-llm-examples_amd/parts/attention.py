@@ -104,7 +104,7 @@ class Attention(Mixer):
         self.output_gate = bool(spec.get("output_gate", False))
         # the path through conv_rows and heads_prepare (see the module's text)
         self.general = (self.maps > 1 or self.output_gate or self.retention[0] == "window_keep"
-                        or ((self.conv_taps > 0 or self.biased or self.value_dim != self.head_dim)
+                        or (not self.spanned and (self.conv_taps > 0 or self.biased or self.value_dim != self.head_dim)
                             and (self.qk_norm_weighted or self.qk_norm_first
                                  or (rot is not None and rot.pairing != "adjacent"))))
         self.lam = None

@@ -47,6 +47,8 @@ def silu(z):
 def causal_conv(u, taps_weight, before=None):
     """u [T, C]; taps_weight [C, K], the last column is the current token's.  ``before``: the K - 1 rows in front of
     the sequence (zeros if None)."""
+    if taps_weight is None:  # (a mixer without a convolution)
+        return u
     T, C = u.shape
     K = taps_weight.shape[1]
     if before is None:
@@ -95,7 +97,8 @@ def turn(x, positions, rot, layout):
 
 
 def visible(i, j, size, keep_first=0):
-    return j <= i and (i - j < size or j < keep_first)
+    """``size`` None: no window."""
+    return j <= i and (size is None or i - j < size or j < keep_first)
 
 
 def masked_softmax(scores, positions, size, keep_first=0):
@@ -109,9 +112,9 @@ def masked_softmax(scores, positions, size, keep_first=0):
 def differential_attention(h, w, p, m, eps, positions):
     T = h.shape[0]
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = causal_conv(h @ w[p + "q"].T, w[p + "q.conv"]).reshape(T, H * 2, dk)
-    k = causal_conv(h @ w[p + "k"].T, w[p + "k.conv"]).reshape(T, G * 2, dk)
-    v = causal_conv(h @ w[p + "v"].T, w[p + "v.conv"]).reshape(T, G, dv)
+    q = causal_conv(h @ w[p + "q"].T, w.get(p + "q.conv")).reshape(T, H * 2, dk)
+    k = causal_conv(h @ w[p + "k"].T, w.get(p + "k.conv")).reshape(T, G * 2, dk)
+    v = causal_conv(h @ w[p + "v"].T, w.get(p + "v.conv")).reshape(T, G, dv)
     q = turn(rms_divide(q, eps) * w[p + "q.norm"], positions, m["rot"], "half")
     k = turn(rms_divide(k, eps) * w[p + "k.norm"], positions, m["rot"], "half")
     lam = (torch.exp((w[p + "lq1"] * w[p + "lk1"]).sum()) - torch.exp((w[p + "lq2"] * w[p + "lk2"]).sum())
@@ -122,7 +125,7 @@ def differential_attention(h, w, p, m, eps, positions):
         a = []
         for mp in range(2):
             sc = (q[:, 2 * hd + mp] @ k[:, 2 * g + mp].T) * m["scale"]
-            a.append(masked_softmax(sc, positions, m["mask"]["size"]) @ v[:, g])
+            a.append(masked_softmax(sc, positions, m.get("mask", {}).get("size")) @ v[:, g])
         o = a[0] - lam * a[1]
         heads.append(rms_divide(o, eps) * (1.0 - m["diff"]))
     o = torch.cat(heads, dim=-1) * torch.sigmoid(h @ w[p + "g"].T)
@@ -140,7 +143,8 @@ def kept_window_attention(h, w, p, m, positions):
     for hd in range(H):
         g = hd // (H // G)
         sc = (q[:, hd] @ k[:, g].T) * m["scale"]
-        heads.append(masked_softmax(sc, positions, m["mask"]["size"], m["mask"].get("keep_first", 0)) @ v[:, g])
+        mask = m.get("mask", {})
+        heads.append(masked_softmax(sc, positions, mask.get("size"), mask.get("keep_first", 0)) @ v[:, g])
     return torch.cat(heads, dim=-1) @ w[p + "o"].T
 
 
@@ -150,9 +154,9 @@ def gated_delta(h, w, p, m, eps, state=None):
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     before = (None, None, None) if state is None else state[1]
     uq, uk, uv = h @ w[p + "q"].T, h @ w[p + "k"].T, h @ w[p + "v"].T
-    q = silu(causal_conv(uq, w[p + "q.conv"], before[0])).reshape(T, G, dk)
-    k = silu(causal_conv(uk, w[p + "k.conv"], before[1])).reshape(T, G, dk)
-    v = silu(causal_conv(uv, w[p + "v.conv"], before[2])).reshape(T, H, dv)
+    q = silu(causal_conv(uq, w.get(p + "q.conv"), before[0])).reshape(T, G, dk)
+    k = silu(causal_conv(uk, w.get(p + "k.conv"), before[1])).reshape(T, G, dk)
+    v = silu(causal_conv(uv, w.get(p + "v.conv"), before[2])).reshape(T, H, dv)
     q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + UNIT_FLOOR) * dk ** -0.5
     k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + UNIT_FLOOR)
     beta = torch.sigmoid(h @ w[p + "b"].T)  # [T, H]
@@ -166,7 +170,7 @@ def gated_delta(h, w, p, m, eps, state=None):
             u = beta[t, hd] * (v[t, hd] - S[hd].T @ k[t, g])
             S[hd] = S[hd] + torch.outer(k[t, g], u)
             out[t, hd] = S[hd].T @ q[t, g]
-    taps = w[p + "q.conv"].shape[1]
+    taps = w[p + "q.conv"].shape[1] if p + "q.conv" in w else 1
     tail = lambda u, b: torch.cat([torch.zeros(taps - 1, u.shape[1], dtype=u.dtype) if b is None else b, u])[-(taps - 1):] \
         if taps > 1 else u[:0]
     o = rms_divide(out, eps) * w[p + "norm"]

@@ -1,0 +1,521 @@
+"""The Sudilorn design in the engine against its plain implementation (``plain_sudilorn.py``): every mechanism alone,
+then whole models however the requests are cut and batched, on the plain ops (CPU) and on the HIP kernels (GPU)."""
+import collections
+import math
+import types
+
+import pytest
+import torch
+
+import plain_sudilorn as P
+import traces
+from jax_llm_examples_amd import Engine, SamplingParams, load_model
+from jax_llm_examples_amd.cache import CacheManager, CacheView
+from jax_llm_examples_amd.config import ConfigError, get_architecture
+from jax_llm_examples_amd.config.specs import part
+from jax_llm_examples_amd.engine import StepEntry, build_context, get_ops
+from jax_llm_examples_amd.engine.replay import make_runner
+from jax_llm_examples_amd.parts.base import build_position, readable
+from jax_llm_examples_amd.parts.residual import ScaledSum
+from sudilorn_configs import SUDILORN, SUDILORN_FAST, draw_sudilorn, sudilorn_config_json, write_sudilorn
+
+DEVICES = [pytest.param("cpu", id="cpu-plain-ops"), pytest.param("cuda:0", id="gpu-hip", marks=pytest.mark.gpu)]
+LENGTHS = {"SA": [1, 80, 33, 47, 64, 9, 130], "SB": [70, 2, 49, 96, 31, 17], "SS": [161, 40, 5, 83],
+           "SF": [420, 40, 170, 33]}
+MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
+TOL = {"float32": 5e-5, "bfloat16": 5e-2}  # of the largest logit of the request
+TOL_OF = {("SS", "bfloat16"): 1.5e-1}  # (sharp scores: a score of 20 rounded by 2^-9 moves its weight by a twentieth)
+
+
+def _ops(device):
+    return get_ops(device, reference_ops=(device == "cpu"))
+
+
+def _load_cpu(folder, dtype="float32"):
+    from jax_llm_examples_amd.engine.loading import load_model as lm
+    return lm(folder, dtype, "cpu")
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("sudilorn")
+    return {name: write_sudilorn(name, str(root / name), torch.float32) for name in SUDILORN}
+
+
+@pytest.fixture(scope="module")
+def folders_bf16(tmp_path_factory):
+    root = tmp_path_factory.mktemp("sudilorn_bf16")
+    return {name: write_sudilorn(name, str(root / name), torch.bfloat16) for name in {**SUDILORN, **SUDILORN_FAST}}
+
+
+# ---------------------------------------------------------------------------------------------- mechanisms alone
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("width", [54, 64, 300, 1000, 2304, 4608, 9000])
+def test_branch_outputs_with_factors_and_the_next_norm(device, width):
+    """x += vector * (fa a + fb b) and the norm of the sum, for one and two terms in either dtype, with and without
+    the vector; then the sum alone."""
+    ops = _ops(device)
+    g = torch.Generator().manual_seed(width)
+    N, D = 5, width
+    d = lambda t: t.to(device)
+    for two, vec, dt in ((True, True, torch.float32), (False, True, torch.bfloat16), (True, False, torch.bfloat16),
+                         (False, False, torch.float32)):
+        x, w = torch.randn(N, D, generator=g), torch.randn(D, generator=g)
+        a, b = torch.randn(N, D, generator=g).to(dt), torch.randn(N, D, generator=g)
+        v = torch.randn(D, generator=g) if vec else None
+        total = 0.7 * a.double() + (-1.3 * b.double() if two else 0.0)
+        want_x = x.double() + (total * v.double() if vec else total)
+        want_h = P.rms_divide(want_x, 1e-5) * w.double()
+        terms = [(d(a), 0.7)] + ([(d(b), -1.3)] if two else [])
+        work = d(x.clone())
+        h, h32 = ops.add_rmsnorm(work, ScaledSum(terms, None if v is None else d(v)), d(w), 1e-5, torch.float32, True)
+        assert torch.allclose(work.cpu().double(), want_x, rtol=1e-5, atol=1e-5)
+        assert torch.allclose(h.cpu().double(), want_h, rtol=1e-4, atol=1e-5) and torch.equal(h, h32)
+        work = d(x.clone())
+        ops.add_residual(work, ScaledSum(terms, None if v is None else d(v)))
+        assert torch.allclose(work.cpu().double(), want_x, rtol=1e-5, atol=1e-5)
+
+
+def test_stretched_rates_of_half_split_pairs():
+    """The position part's rates and magnitude are the plain formula's, with ramps that start before the first pair,
+    end beyond the last, or have no width."""
+    for base, dims, sc in ((250000.0, 32, (4.0, 2048, 32.0, 1.0)), (5000.0, 12, (8.0, 64, 4.0, 1.0)),
+                           (30.0, 6, (4.0, 16, 8.0, 2.0)), (10000.0, 8, (2.0, 32, 2.0, 2.0)), (100.0, 8, None)):
+        rot = {"base": base, "dims": dims}
+        if sc is not None:
+            rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), sc))
+        rates, grow = P.rotary_rates(rot)
+        r = build_position(part("rope_yarn", theta=base, rotary_dim=dims, scaling=sc, pairing="half"), dims + 4).rotation()
+        assert r.pairing == "half" and r.rotary_dim == dims and abs(r.magnitude - grow) < 1e-12
+        assert torch.allclose(r.inv_freq.double(), torch.tensor(rates, dtype=torch.float64), rtol=1e-6, atol=0)
+
+
+def test_window_with_kept_first_tokens_as_a_rule():
+    for W, K in ((5, 2), (3, 9), (16, 1)):
+        for i in range(60):
+            for j in range(60):
+                assert readable(("window_keep", W, K), i, j) == P.visible(i, j, W, K)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("experts,top,groups,keep", [(8, 3, 2, 1), (6, 2, 3, 2), (4, 4, None, None), (12, 2, 12, 3),
+                                                     (5, 1, 1, 1), (16, 4, 4, 2)])
+def test_choice_of_experts_alone(device, experts, top, groups, keep):
+    """Scores, a correction that makes choice scores negative, groups scored by their two largest, ties by index."""
+    ops = _ops(device)
+    g = torch.Generator().manual_seed(experts * 7 + top)
+    D, N = 24, 40
+    h = torch.randn(N, D, generator=g)
+    router = torch.randn(experts, D, generator=g) * 0.5
+    correction = torch.randn(experts, generator=g) * 0.8 - 1.0
+    ids, wts, _ = ops.moe_choose(h.to(device), router.to(device), correction.to(device), top, groups, keep, 2)
+    cfg = {"experts": experts, "top": top}
+    if groups is not None:
+        cfg["groups"] = {"count": groups, "keep": keep}
+    z = h.double() @ router.double().T
+    for t in range(N):
+        want_ids, want_w = P.choose_experts(z[t], correction.double(), cfg)
+        assert ids[t].tolist() == want_ids, (t, ids[t].tolist(), want_ids)
+        assert torch.allclose(wts[t].cpu().double(), torch.stack(want_w), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,layer", [("SA", 0), ("SA", 1), ("SA", 3), ("SB", 0), ("SB", 1), ("SB", 3), ("SS", 1)])
+def test_scored_experts_alone(folders, device, name, layer):
+    cfg, w = P.load(folders[name])
+    model = load_model(folders[name], "float32", device) if device != "cpu" else _load_cpu(folders[name])
+    ff = model.blocks[layer].feed_forward
+    h = torch.randn(23, cfg["width"], generator=torch.Generator().manual_seed(layer))
+    wd = {k: v.double() for k, v in w.items() if v.is_floating_point()}
+    want, _ = P.routed_experts(h.double(), wd, f"l{layer}.mlp.", cfg["layers"][layer]["mlp"])
+    ctx = types.SimpleNamespace(ops=_ops(device), tap=None, dtype=torch.float32)
+    got = ctx.ops.materialize(ff.forward(h.to(device), h.to(device), ctx)).float().cpu()
+    assert torch.allclose(got, want.float(), rtol=2e-4, atol=2e-5), (got - want.float()).abs().max()
+
+
+def _mixer_alone(folder, device, layer, sizes, x, dtype="float32", page_size=16, change=None):
+    """Runs one layer's mixer over the paged cache and its per-request state in the given portions."""
+    model = load_model(folder, dtype, device) if device != "cpu" else _load_cpu(folder, dtype)
+    ops = _ops(device)
+    mixer = model.blocks[layer].mixer
+    if change is not None:
+        change(mixer)
+    pages = -(-sum(sizes) // page_size) + 1
+    cache = CacheManager({0: mixer.cache_need()}, page_size=page_size, num_pages=pages, max_requests=1, dtype=model.dtype,
+                         device=device, poison=True)
+    outs, o = [], 0
+    for n in sizes:
+        if not cache.has_request("r"):
+            cache.add_request("r")
+        cache.reserve("r", n)
+        ctx = build_context(ops, model.dtype, device, cache, [StepEntry("r", [0] * n, [])], model.config.vocab)
+        view = CacheView(0, True, state=cache.state.get(0), states=cache.named_state.get(0))
+        if cache.groups:
+            gctx = ctx.groups[0]
+            view = CacheView(0, True, kv=cache.groups[0].tensors.get(0), block_table=gctx.block_table,
+                             slot_mapping=gctx.slot_mapping, attn_meta=gctx, group=0, pages=cache.groups[0].pages[0],
+                             state=cache.state.get(0), states=cache.named_state.get(0))
+        h = x[o:o + n].to(device)
+        if getattr(mixer, "wants_float32_input", False):
+            y = mixer.forward(h.to(model.dtype), ctx, view, h)
+        else:
+            y = mixer.forward(h.to(model.dtype), ctx, view)
+        outs.append(ops.materialize(y).float().cpu())
+        cache.commit("r")
+        o += n
+    return torch.cat(outs)
+
+
+def _plain_mixer(cfg, w, layer, x, change=None):
+    lc, eps, p = cfg["layers"][layer], cfg["norm"]["eps"], f"l{layer}.mix."
+    wd = {k: v.double() for k, v in w.items() if v.is_floating_point()}
+    if change is not None:
+        change(wd, p)
+    pos = list(range(x.shape[0]))
+    if lc["type"] == "attention":
+        return P.differential_attention(x.double(), wd, p, lc["mixer"], eps, pos).float()
+    return P.parallel_mixer(x.double(), wd, p, lc["mixer"], eps, pos).float()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,layer", [("SA", 0), ("SA", 1), ("SA", 2), ("SA", 3), ("SB", 0), ("SB", 1), ("SB", 2),
+                                        ("SB", 3), ("SS", 0), ("SS", 1)])
+def test_mixers_alone(folders, device, name, layer):
+    """Each mixer whole, in portions down to two tokens and token by token (also the first tokens of a sequence one
+    by one: shorter than the convolution's taps) equals the plain mixer."""
+    cfg, w = P.load(folders[name])
+    T = 75
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(layer + 1))
+    want = _plain_mixer(cfg, w, layer, x)
+    for sizes in ([T], [30, 2, 17, 1, 1, 24], [1] * T):
+        got = _mixer_alone(folders[name], device, layer, sizes, x)
+        assert torch.allclose(got, want, rtol=3e-4, atol=3e-5), (sizes[:3], (got - want).abs().max())
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_delta_rule_long_decoding_through_both_halves_of_its_state(folders, device):
+    """Hundreds of single tokens; inputs large enough that decays and write strengths reach both their ends."""
+    name, layer = "SB", 2  # (its left mixer has no window: every key stays)
+    cfg, w = P.load(folders[name])
+    T = 300
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(3)) * 3.0
+    want = _plain_mixer(cfg, w, layer, x)
+    for sizes in ([T], [3] + [1] * (T - 3), [149, 2, 149]):
+        got = _mixer_alone(folders[name], device, layer, sizes, x)
+        assert torch.allclose(got, want, rtol=5e-4, atol=5e-5), (got - want).abs().max()
+
+
+def _sharpen_left(mixer):
+    """The left attention's keys are projected with its first query heads' matrix and no bias is left: a token that
+    has the direction of the last one then takes the last query's weight, if the query may see it."""
+    a = mixer.left
+    nq, nk = a.num_heads * a.head_dim, a.num_kv_heads * a.head_dim
+    a.params["wqkv"][nq:nq + nk].copy_(a.params["wqkv"][:nk])
+    a.params["bqkv"].zero_()
+    a.finalize()
+    mixer.right.params["wo"].zero_()  # (the attention alone)
+
+
+def _sharpen_left_plain(wd, p):
+    nk = wd[p + "left.k"].shape[0]
+    wd[p + "left.k"] = wd[p + "left.q"][:nk].clone()
+    for n in ("q", "k", "v"):
+        wd[p + f"left.{n}.b"] = torch.zeros_like(wd[p + f"left.{n}.b"])
+    wd[p + "right.o"] = torch.zeros_like(wd[p + "right.o"])
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("decoding", [False, True])
+@pytest.mark.parametrize("back", ["first", "last_kept", "first_not_kept", "just_outside", "just_inside", "page_edge"])
+def test_one_key_that_stands_out_at_the_windows_edges(folders, device, decoding, back):
+    """One early token is given the last token's direction.  Where it is the first token, the last kept one, or just
+    inside the window, the last query's weight lies on it; where it is the first token that is not kept, or just
+    outside the window, the query does not see it: the plain mixer says which, and the engine follows it, in a prompt
+    and in decoding, hundreds of tokens back."""
+    name, layer = "SS", 0  # window 48, the first 2 tokens kept
+    cfg, w = P.load(folders[name])
+    W, K = 48, 2
+    T = 290
+    special = {"first": 0, "last_kept": K - 1, "first_not_kept": K, "just_outside": T - 1 - W, "just_inside": T - W,
+               "page_edge": T - 1 - 31}[back]
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(9))
+    x[special] = 3.0 * x[T - 1]
+    want = _plain_mixer(cfg, w, layer, x, change=_sharpen_left_plain)
+    sizes = [special + 3] + [1] * (T - special - 3) if decoding else [T]
+    got = _mixer_alone(folders[name], device, layer, sizes, x, change=_sharpen_left)
+    assert torch.allclose(got, want, rtol=5e-4, atol=5e-5), (got - want).abs().max()
+    x2 = x.clone()
+    x2[special] = torch.randn(cfg["width"], generator=torch.Generator().manual_seed(1))
+    moved = (_plain_mixer(cfg, w, layer, x2, change=_sharpen_left_plain)[T - 1] - want[T - 1]).abs().max()
+    assert (moved > 1e-2) == (back not in ("first_not_kept", "just_outside")), moved
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("decoding", [False, True])
+def test_two_score_maps_with_sharp_scores_at_the_windows_edge(folders, device, decoding):
+    """The q/k norms' weights are made large, so that each map's weight lies on few keys: a window that is one token
+    off, or a map that reads the other's keys, then changes the output by much more than the tolerance."""
+    name, layer = "SS", 1  # window 37, taps 3
+    cfg, w = P.load(folders[name])
+    T = 200
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(11))
+
+    def change(mixer):
+        mixer.params["q_norm"].mul_(4.0)
+        mixer.params["k_norm"].mul_(3.0)
+
+    def change_plain(wd, p):
+        wd[p + "q.norm"] = wd[p + "q.norm"] * 4.0
+        wd[p + "k.norm"] = wd[p + "k.norm"] * 3.0
+
+    want = _plain_mixer(cfg, w, layer, x, change=change_plain)
+    sizes = [80] + [1] * (T - 80) if decoding else [T]
+    got = _mixer_alone(folders[name], device, layer, sizes, x, change=change)
+    assert torch.allclose(got, want, rtol=1e-3, atol=1e-4), (got - want).abs().max()
+    one_off = dict(cfg["layers"][layer]["mixer"], mask={"size": 36})
+    wd = {k: v.double() for k, v in w.items() if v.is_floating_point()}
+    change_plain(wd, f"l{layer}.mix.")
+    other = P.differential_attention(x.double(), wd, f"l{layer}.mix.", one_off, cfg["norm"]["eps"], list(range(T))).float()
+    assert (other - want).abs().max() > 1e-2
+
+
+# ---------------------------------------------------------------------------------------------- whole models
+def _plain_logits(folder, toks, choices=None):
+    cfg, w = P.load(folder)
+    table = None
+    if choices is not None:
+        table = [choices.get(i) for i in range(len(cfg["layers"]))]
+    return P.forward(cfg, w, toks, choices=table)[0].float()
+
+
+def _check(name, folder, dtype, device, mode, record=False, page_size=16, lengths=None, top=None, seed=5):
+    lengths = lengths or (LENGTHS[name] + (LENGTHS[name][::-1] if mode == "mixed" else []))
+    vocab = (top or sudilorn_config_json(name))["vocab"]
+    reqs = traces.random_requests(vocab, lengths, seed=seed)
+    steps = MODES[mode](reqs)
+    runner = make_runner(folder, dtype, traces.max_live_tokens(steps), device, reference_ops=(device == "cpu"),
+                         poison=True, max_requests=4, page_size=page_size, decode_graphs=None if record else False)
+    handed = [collections.Counter() for _ in runner.cache.groups]
+    for g, seen in zip(runner.cache.groups, handed):
+        def alloc(n, inner=g.pool.alloc, seen=seen):
+            pages = inner(n)
+            seen.update(pages)
+            return pages
+        g.pool.alloc = alloc
+    # (in bfloat16 a router's close call may fall the other way: the plain model is then told the engine's choices,
+    # and still forms the scores itself)
+    routes = {}
+    if dtype == "bfloat16":
+        got, routes = traces.run_trace(runner, steps, record_routing=True)
+    else:
+        got = traces.run_trace(runner, steps)
+    if record:
+        assert runner.graphs is not None and runner.graphs.replays > 0
+    if mode == "mixed" and top is None:  # pages and slots were used again
+        assert all(max(seen.values()) > 1 for seen in handed)
+        assert len(reqs) > runner.cache.max_requests
+    runner.cache.check()
+    assert runner.cache.num_live() == 0 and all(g.pool.num_held == 0 for g in runner.cache.groups)
+    for rid, toks in reqs.items():
+        choices = {li: ids.long() for li, ids in routes[rid].items()} if rid in routes else None
+        ref = _plain_logits(folder, toks, choices)
+        assert got[rid].shape == ref.shape and torch.isfinite(got[rid]).all(), f"{rid}: non-finite logits"
+        err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
+        bad = (err > TOL_OF.get((name, dtype), TOL[dtype])).nonzero().squeeze(-1).tolist()
+        assert not bad, f"{name} {dtype} {mode} {rid}: first wrong position {bad[0]} of {len(toks)}, error {err[bad[0]]:.3g}"
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(SUDILORN))
+def test_cpu_plain_ops_float32(folders, name, mode):
+    _check(name, folders[name], "float32", "cpu", mode)
+
+
+@pytest.mark.parametrize("page_size", [4, 64])
+def test_cpu_other_page_sizes(folders, page_size):
+    _check("SA", folders["SA"], "float32", "cpu", "mixed", page_size=page_size)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(SUDILORN))
+def test_gpu_float32(folders, name, mode):
+    _check(name, folders[name], "float32", "cuda:0", mode)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["tail", "mixed"])
+@pytest.mark.parametrize("name", list(SUDILORN))
+def test_gpu_float32_with_recorded_decode_steps(folders, name, mode):
+    _check(name, folders[name], "float32", "cuda:0", mode, record=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(SUDILORN) + list(SUDILORN_FAST))
+def test_gpu_bfloat16(folders_bf16, name, mode):
+    _check(name, folders_bf16[name], "bfloat16", "cuda:0", mode)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("page_size", [4, 64])
+def test_gpu_other_page_sizes(folders, page_size):
+    _check("SA", folders["SA"], "float32", "cuda:0", "mixed", page_size=page_size)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["SA", "SB", "SF"])
+def test_gpu_bfloat16_recorded_decode_steps_equal_unrecorded_ones(folders_bf16, name):
+    """Steps of single tokens replayed from recorded graphs give the bits of the same steps run launch by launch:
+    the memory's two halves, the convolutions' rows and the pages are those of the step, not of the recording."""
+    reqs = traces.random_requests(sudilorn_config_json(name)["vocab"], [90, 41, 67], seed=6)
+    steps = traces.tail(reqs, last=40)
+    outs = []
+    for graphs in (None, False):
+        runner = make_runner(folders_bf16[name], "bfloat16", traces.max_live_tokens(steps), "cuda:0", poison=True,
+                             max_requests=4, decode_graphs=graphs)
+        outs.append(traces.run_trace(runner, steps))
+        if graphs is None:
+            assert runner.graphs is not None and runner.graphs.replays > 0
+    for rid in reqs:
+        assert torch.equal(outs[0][rid], outs[1][rid])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(SUDILORN_FAST))
+def test_gpu_float32_at_vector_sizes(tmp_path, name):
+    folder = write_sudilorn(name, str(tmp_path / name), torch.float32)
+    for mode in ("portions", "mixed"):
+        _check(name, folder, "float32", "cuda:0", mode)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_gpu_configurations_drawn_at_random(tmp_path, seed, dtype):
+    from jax_llm_examples_amd.weights import write_random_model
+
+    top, page_size, lengths = draw_sudilorn(seed)
+    arch = get_architecture("Sudilorn")
+    folder = write_random_model(arch, arch.parse_config(top), str(tmp_path / "m"), seed,
+                                torch.float32 if dtype == "float32" else torch.bfloat16)
+    _check("drawn", folder, dtype, "cuda:0", "mixed", page_size=page_size, lengths=lengths, top=top, seed=seed)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_cpu_configurations_drawn_at_random(tmp_path, seed):
+    from jax_llm_examples_amd.weights import write_random_model
+
+    top, page_size, lengths = draw_sudilorn(seed)
+    arch = get_architecture("Sudilorn")
+    folder = write_random_model(arch, arch.parse_config(top), str(tmp_path / "m"), seed, torch.float32)
+    _check("drawn", folder, "float32", "cpu", "mixed", page_size=page_size, lengths=lengths, top=top, seed=seed)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name", ["SA", "SB"])
+def test_residual_stream_behind_every_layer(folders, device, name):
+    """What a watcher of the step sees behind every layer equals the plain model's stream."""
+    folder = folders[name]
+    cfg, w = P.load(folder)
+    toks = traces.random_requests(128, [29], seed=2)["r0"]
+    want = []
+    P.forward(cfg, w, toks, taps=want)
+    runner = make_runner(folder, "float32", 64, device, reference_ops=(device == "cpu"), max_requests=2)
+    seen = []
+    runner.step([StepEntry("r", toks, [])], tap=lambda part_, nm, value: seen.append(value()) if nm == "residual" else None)
+    assert len(seen) == len(want) == len(cfg["layers"])
+    for a, b in zip(seen, want):
+        assert torch.allclose(a.cpu(), b.float(), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_a_token_far_back_matters_through_the_memory_alone(folders, device, tmp_path):
+    """Both layers' windows end long before it, and the first tokens that stay are not it: the logits at the last token
+    still change with a token 150 places back, through the delta rule's memory (whose decay is made slow); the engine
+    follows the plain model in a prompt and in decoding."""
+    import os
+    import shutil
+
+    from safetensors.torch import save_file
+
+    folder = str(tmp_path / "slow")
+    shutil.copytree(folders["SS"], folder)
+    _, w = P.load(folder)
+    w["l0.mix.right.A_log"] = torch.full_like(w["l0.mix.right.A_log"], -7.0)
+    save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(folder, "model.safetensors"))
+    toks = traces.random_requests(128, [170], seed=4)["r0"]
+    i = 169
+
+    def logits_at(seq, decoding):
+        runner = make_runner(folder, "float32", 256, device, reference_ops=(device == "cpu"), max_requests=2)
+        if not decoding:
+            runner.step([StepEntry("r", seq[:i], [])])
+            return runner.step([StepEntry("r", seq[i:i + 1], [0])])[0].cpu().clone()
+        runner.step([StepEntry("r", seq[:140], [])])
+        for t in range(140, i):
+            runner.step([StepEntry("r", [seq[t]], [])])
+        return runner.step([StepEntry("r", [seq[i]], [0])])[0].cpu().clone()
+
+    other = list(toks)
+    other[19] = (toks[19] + 1) % 128
+    for decoding in (False, True):
+        a, b = logits_at(toks, decoding), logits_at(other, decoding)
+        wa, wb = _plain_logits(folder, toks)[i], _plain_logits(folder, other)[i]
+        assert (wa - wb).abs().max() > 1e-3
+        assert torch.allclose(a, wa, rtol=5e-5, atol=5e-5) and torch.allclose(b, wb, rtol=5e-5, atol=5e-5)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_the_engine(folders, device):
+    """``Engine.generate`` with its scheduler (portions of prompts beside decoded tokens, four requests at a time)
+    gives the plain model's greedy tokens."""
+    name = "SA"
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, 300, (n,), generator=g).tolist() for n in (7, 40, 19, 3, 55)]
+    steps = 10
+    want = []
+    for p in prompts:
+        seq = list(p)
+        for _ in range(steps):
+            seq.append(int(_plain_logits(folders[name], seq)[-1].argmax()))
+        want.append(seq[len(p):])
+    model = load_model(folders[name], "float32", device) if device != "cpu" else _load_cpu(folders[name])
+    engine = Engine(model, cache_tokens=512, decode_batch_size=4, max_num_batched_tokens=24,
+                    **({"reference_ops": True} if device == "cpu" else {}))
+    got = engine.generate(prompts, SamplingParams(max_decode_length=steps))
+    assert got == want
+
+
+# ---------------------------------------------------------------------------------------------- configuration
+def test_configuration_round_trip_and_errors():
+    arch = get_architecture("Sudilorn")
+    for name in list(SUDILORN) + list(SUDILORN_FAST):
+        top = sudilorn_config_json(name)
+        cfg = arch.parse_config(top)
+        assert arch.parse_config(arch.config_to_dict(cfg)) == cfg
+        assert len(arch.plan(cfg).layers) == len(top["layers"])
+    for seed in range(30):
+        top, _, _ = draw_sudilorn(seed)
+        cfg = arch.parse_config(top)
+        assert arch.parse_config(arch.config_to_dict(cfg)) == cfg
+    bad = sudilorn_config_json("SA")
+    bad["layers"][0]["mlp"]["router"]["groups"] = {"count": 4, "keep": 1}  # (six experts in four groups)
+    with pytest.raises(ConfigError):
+        arch.parse_config(bad)
+    bad = sudilorn_config_json("SA")
+    bad["layers"][1]["mixer"]["mask"]["keep_first"] = 2  # (a key this mixer does not have)
+    with pytest.raises(ConfigError):
+        arch.parse_config(bad)
+    bad = sudilorn_config_json("SA")
+    bad["layers"][1]["mixer"]["rot"]["dims"] = 18  # (more turned elements than a head has)
+    with pytest.raises(ConfigError):
+        arch.parse_config(bad)
+    bad = sudilorn_config_json("SA")
+    bad["layers"][2]["type"] = "gru"
+    with pytest.raises(ConfigError):
+        arch.parse_config(bad)
+    bad = sudilorn_config_json("SA")
+    bad["layers"][3]["mlp"]["router"]["top"] = 5  # (the one group that stays holds four experts)
+    with pytest.raises(ConfigError):
+        arch.parse_config(bad)
