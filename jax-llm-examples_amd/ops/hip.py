@@ -695,7 +695,12 @@ class HipOps:
         return h.rows(want32) if isinstance(h, PendingNorm) else h
 
     def materialize(self, delta):
-        """The tensor an :class:`ExpertSum` stands for (float32); anything else as it is."""
+        """The tensor an :class:`ExpertSum` (or a sum with factors) stands for (float32); anything else as it is."""
+        if hasattr(delta, "terms"):
+            first = delta.terms[0][0]
+            total = torch.zeros(first.shape[0], first.shape[1], dtype=torch.float32, device=self.device)
+            self.scaled_add_norm(total, delta, None, 0.0, torch.float32, norm=False)
+            return total
         if not isinstance(delta, ExpertSum):
             return delta
         n, d = delta.shape
