@@ -89,7 +89,23 @@ def design_configs(size: dict, layers: int):
                "embedding": {"scale": 1.0}, "streams": 4, "layers": m_layers}
     llama_moe = dict(llama, interleave_moe_layer_step=1, moe_layers=list(range(layers)), num_local_experts=8,
                      num_experts_per_tok=1, intermediate_size=size["ff"] // 2)
-    return {"rovidra": rovidra, "tiradra": tiradra, "llama4-dense": llama, "mazotar": mazotar, "llama4-moe": llama_moe}
+    # Sudilorn: two layers of an attention (window with kept first tokens) beside a gated-delta-rule memory, then one
+    # of attention with two score maps per head (half the heads, values twice as wide), and so on; eight scored
+    # experts in four groups, two a token; its closest model here is the same Llama 4 with routed layers
+    s_left = {"heads": size["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+              "mask": {"size": size["span"], "keep_first": 4}, "rot": {"base": 500000.0, "dims": 64}}
+    s_right = {"heads": size["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "conv": 4}
+    s_diff = {"heads": size["heads"] // 2, "kv_heads": 4, "dim": 128, "vdim": 256, "scale": 128 ** -0.5, "diff": 0.6,
+              "conv": 4, "mask": {"size": size["span"]}, "rot": {"base": 500000.0, "dims": 64, "scaling": yarn}}
+    s_moe = {"kind": "moe", "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}},
+             "expert": {"ff": size["ff"] // 2}}
+    sudilorn = {"architecture": "Sudilorn", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-5},
+                "residual_mult": 0.5,
+                "layers": [{"type": "attention", "mixer": s_diff, "mlp": s_moe} if i % 3 == 2 else
+                           {"type": "parallel", "mixer": {"left": s_left, "right": s_right, "left_scale": 0.8,
+                                                          "right_scale": 0.5}, "mlp": s_moe} for i in range(layers)]}
+    return {"rovidra": rovidra, "tiradra": tiradra, "llama4-dense": llama, "mazotar": mazotar, "llama4-moe": llama_moe,
+            "sudilorn": sudilorn}
 
 
 def bench_designs(args) -> int:
@@ -198,10 +214,10 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--design-points", default="1@2048,8@2048,64@2048", help="decode steps of --designs: batch@context")
     ap.add_argument("--designs", default="", help="instead of the default workload: prefill and decode of the Rovidra, "
-                    "Tiradra and Mazotar designs beside the Llama 4 layers of equal sizes, at the named sizes "
+                    "Tiradra, Mazotar and Sudilorn designs beside the Llama 4 layers of equal sizes, at the named sizes "
                     "(comma-separated, of " + ", ".join(DESIGN_SIZES) + "; 'all')")
     ap.add_argument("--design-names", default="", help="with --designs: only these of rovidra, tiradra, llama4-dense, "
-                    "mazotar, llama4-moe")
+                    "mazotar, llama4-moe, sudilorn")
     args = ap.parse_args()
     if args.designs:
         return bench_designs(args)

@@ -257,7 +257,7 @@ __device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], con
                                             const int* __restrict__ table, const Columns (&col)[CT], int k_lo,
                                             int k_hi, int hk, int Hkv, int ps, float scale_log2, float (&m)[CT],
                                             float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad,
-                                            Biasing bias = Biasing{nullptr, 0}) {
+                                            Biasing bias = Biasing{nullptr, 0}, bool fresh = true, bool close = true) {
   const int lane = threadIdx.x & 63;
   const int c16 = lane & 15, g = lane >> 4;
   constexpr int KC = DH / 32;  // k-steps of the first product
@@ -265,12 +265,15 @@ __device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], con
   const size_t plane = (size_t)ps * DH;
   const size_t page_stride = 2 * (size_t)Hkv * plane;
 
+  // (fresh = false: the sums go on from what another range of keys left, which was not closed)
+  if (fresh) {
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    m[ct] = -INFINITY;
-    l[ct] = 0.f;
+    for (int ct = 0; ct < CT; ++ct) {
+      m[ct] = -INFINITY;
+      l[ct] = 0.f;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
   }
 
   // The keys and values of a step are asked for one step ahead: they are in registers when the step begins.
@@ -393,8 +396,10 @@ __device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], con
     else
       softmax_and_values<DH, CT, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
   }
+  if (close) {
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) l[ct] = column_sum(l[ct]);
+    for (int ct = 0; ct < CT; ++ct) l[ct] = column_sum(l[ct]);
+  }
 }
 
 template <int DH, int CT, bool ONCE, bool BIASED = false>
@@ -402,10 +407,11 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
                                        const int* __restrict__ table, const Columns (&col)[CT], int k_lo, int k_hi,
                                        int hk, int Hq, int Hkv, int ps, float scale_log2, float (&m)[CT],
                                        float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad,
-                                       Biasing bias = Biasing{nullptr, 0}) {
+                                       Biasing bias = Biasing{nullptr, 0}, bool fresh = true, bool close = true) {
   bf16x8 qb[CT][DH / 32];
   load_queries<DH, CT>(q, col, Hq, qb);
-  attend_with<DH, CT, ONCE, BIASED>(qb, kv, table, col, k_lo, k_hi, hk, Hkv, ps, scale_log2, m, l, acc, bad, bias);
+  attend_with<DH, CT, ONCE, BIASED>(qb, kv, table, col, k_lo, k_hi, hk, Hkv, ps, scale_log2, m, l, acc, bad, bias,
+                                    fresh, close);
 }
 
 // ------------------------------------------------------------------ prefill portions
@@ -453,6 +459,66 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128 && !BIASED) ? 2 : 1) voi
   for (int ct = 0; ct < CT; ++ct) {
     if (ct * 16 + c16 >= nt) continue;
     if (BIASED && sink != nullptr) l[ct] += exp2f(sink[h] * kLog2e - m[ct]);
+    const float inv = bad ? __builtin_nanf("") : (l[ct] > 0.f ? 1.0f / l[ct] : 0.f);
+    bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt) {
+      const uint2 v = {pack_bf16(acc[ct][dt][0] * inv, acc[ct][dt][1] * inv),
+                       pack_bf16(acc[ct][dt][2] * inv, acc[ct][dt][3] * inv)};
+      *reinterpret_cast<uint2*>(o + dt * 16) = v;
+    }
+  }
+}
+
+// The same for a window whose queries also see the sequence's first `keep` keys: those of them that lie before a
+// column's window are a range of their own, attended first; the window's keys then go on from its sums.
+template <int DH, int CT>
+__global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention_prefill_kept_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
+    const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
+    int table_width, const int* __restrict__ tiles, int num_tiles, int window, int keep, float scale_log2, int Hq,
+    int Hkv, int ps) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + wave_index();
+  if (item >= num_tiles * Hq) return;
+  const int tile = num_tiles - 1 - item / Hq, h = item % Hq;
+  const int n0 = tiles[2 * tile], nt = tiles[2 * tile + 1];
+  const int hk = h / (Hq / Hkv);
+  const int c16 = lane & 15, g = lane >> 4;
+  const int p_first = positions[n0], p_last = p_first + nt - 1;
+  const int k_lo = first_key(2, window, p_first), k_hi = p_last;
+  const int kept_hi = min(keep, first_key(2, window, p_last)) - 1;  // the last kept key that any column takes apart
+  Columns col[CT], kept[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = ct * 16 + c16;
+    const bool ok = c < nt;
+    const int pos = p_first + c;
+    col[ct].token = ok ? n0 + c : n0;
+    col[ct].head = h;
+    col[ct].lo = ok ? first_key(2, window, pos) : 1;
+    col[ct].hi = ok ? pos : 0;
+    col[ct].pos = pos;
+    kept[ct] = col[ct];
+    kept[ct].lo = ok ? 0 : 1;
+    kept[ct].hi = ok ? min(keep, col[ct].lo) - 1 : 0;
+  }
+  float m[CT], l[CT];
+  f32x4 acc[CT][DH / 16];
+  bool bad = false;
+  const int* table = block_table + (size_t)token_segment[n0] * table_width;
+  if (kept_hi >= 0) {
+    attend<DH, CT, false, false>(q, kv, table, kept, 0, kept_hi, hk, Hq, Hkv, ps, scale_log2, m, l, acc, bad,
+                                 Biasing{nullptr, 0}, true, false);
+    attend<DH, CT, false, false>(q, kv, table, col, k_lo, k_hi, hk, Hq, Hkv, ps, scale_log2, m, l, acc, bad,
+                                 Biasing{nullptr, 0}, false, true);
+  } else {
+    attend<DH, CT, false, false>(q, kv, table, col, k_lo, k_hi, hk, Hq, Hkv, ps, scale_log2, m, l, acc, bad);
+  }
+  bad = __any(bad);
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (ct * 16 + c16 >= nt) continue;
     const float inv = bad ? __builtin_nanf("") : (l[ct] > 0.f ? 1.0f / l[ct] : 0.f);
     bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
 #pragma unroll
@@ -1552,6 +1618,40 @@ JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, cons
   }
 #undef LAUNCH
 #undef LAUNCH_B
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
+// A window of `window` keys whose queries also see the sequence's first `keep` keys; tiles of 16 or 32 tokens, one
+// wavefront per (tile, query head).
+JLE_API int jle_attention_prefill_kept(const void* q, const void* kv, void* out, const int* positions,
+                                       const int* token_segment, const int* block_table, int table_width,
+                                       const int* tiles, int num_tiles, int tile_tokens, int window, int keep,
+                                       float scale, int Hq, int Hkv, int dh, int ps, hipStream_t s) {
+  if (num_tiles <= 0) return 0;
+  if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps)) return JLE_BAD_ARG;
+  if (window <= 0 || keep < 0 || (tile_tokens != 16 && tile_tokens != 32)) return JLE_BAD_ARG;
+  const long long items = (long long)num_tiles * Hq;
+  dim3 g((unsigned)((items + 3) / 4)), b(256);
+  const float sl = scale * kLog2e;
+#define LAUNCH_K(DH, CT)                                                                                             \
+  hipLaunchKernelGGL((attention_prefill_kept_kernel<DH, CT>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,       \
+                     (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles, window,     \
+                     keep, sl, Hq, Hkv, ps)
+#define LAUNCH(DH)                       \
+  do {                                   \
+    if (tile_tokens == 32) LAUNCH_K(DH, 2); \
+    else LAUNCH_K(DH, 1);                \
+  } while (0)
+  switch (dh) {
+    case 32: LAUNCH(32); break;
+    case 64: LAUNCH(64); break;
+    case 96: LAUNCH(96); break;
+    case 128: LAUNCH(128); break;
+    case 256: LAUNCH(256); break;
+  }
+#undef LAUNCH
+#undef LAUNCH_K
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -71,40 +71,53 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   float S[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) S[i] = (live && k0 + i < dk) ? s_old[(size_t)(k0 + i) * dv + c] : 0.f;
-  float kq[2][R], qq[2][R], vv[2], bb[2], gg[2];
-  auto fetch = [&](int t, int buf) {
+  // this token's rows and the next one's, each in registers of its own (asked for a token ahead)
+  float kc[R], qc[R], vc = 0.f, bc = 0.f, gc = 1.f;
+  auto fetch = [&](int t, float (&k_)[R], float (&q_)[R], float& v_, float& b_, float& g_) {
     const float* kp = kn + ((size_t)t * G + g) * dk + k0;
     const float* qp = qn + ((size_t)t * G + g) * dk + k0;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-      kq[buf][i] = k0 + i < dk ? kp[i] : 0.f;
-      qq[buf][i] = k0 + i < dk ? qp[i] : 0.f;
+      k_[i] = k0 + i < dk ? kp[i] : 0.f;
+      q_[i] = k0 + i < dk ? qp[i] : 0.f;
     }
-    vv[buf] = live ? Num<T>::load(rows + (size_t)t * C + 2 * G * dk + (size_t)h * dv + c) : 0.f;
-    bb[buf] = beta[(size_t)t * H + h];
-    gg[buf] = decay[(size_t)t * H + h];
+    v_ = live ? Num<T>::load(rows + (size_t)t * C + 2 * G * dk + (size_t)h * dv + c) : 0.f;
+    b_ = beta[(size_t)t * H + h];
+    g_ = decay[(size_t)t * H + h];
   };
-  if (t0 < t1) fetch(t0, 0);
+  if (t0 < t1) fetch(t0, kc, qc, vc, bc, gc);
   for (int t = t0; t < t1; ++t) {
-    const int cur = (t - t0) & 1;
-    if (t + 1 < t1) fetch(t + 1, cur ^ 1);
-    const float gt = gg[cur];
+    float kx[R], qx[R], vx = 0.f, bx = 0.f, gx = 1.f;
+    if (t + 1 < t1) {
+      fetch(t + 1, kx, qx, vx, bx, gx);
+    } else {
+#pragma unroll
+      for (int i = 0; i < R; ++i) kx[i] = qx[i] = 0.f;
+    }
     float dot = 0.f;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-      S[i] *= gt;
-      dot = __builtin_fmaf(S[i], kq[cur][i], dot);
+      S[i] *= gc;
+      dot = __builtin_fmaf(S[i], kc[i], dot);
     }
     for (int o = cols; o < 64; o <<= 1) dot += __shfl_xor(dot, o, 64);
-    const float u = bb[cur] * (vv[cur] - dot);
+    const float u = bc * (vc - dot);
     float out = 0.f;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-      S[i] = __builtin_fmaf(kq[cur][i], u, S[i]);
-      out = __builtin_fmaf(S[i], qq[cur][i], out);
+      S[i] = __builtin_fmaf(kc[i], u, S[i]);
+      out = __builtin_fmaf(S[i], qc[i], out);
     }
     for (int o = cols; o < 64; o <<= 1) out += __shfl_xor(out, o, 64);
     if (live && ks == 0) o_raw[((size_t)t * H + h) * dv + c] = out;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      kc[i] = kx[i];
+      qc[i] = qx[i];
+    }
+    vc = vx;
+    bc = bx;
+    gc = gx;
   }
   if (live) {
 #pragma unroll

@@ -97,6 +97,7 @@ _SIGNATURES = {
     "jle_moe_choose": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_relu2": [_vp, _vp, _i, _ll, _vp],
     "jle_conv_rows_act": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "jle_attention_prefill_kept": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_paged_attention_kept": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                                  _vp, _vp],
     "jle_paged_attention_biased": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
@@ -1545,6 +1546,28 @@ class HipOps:
         if dh % 8 or dh > 256 or hq % hk:
             raise KernelError(f"attention kernels: head size {dh} (a multiple of 8, at most 256) or {hq} query heads "
                               f"on {hk} kv heads are not supported")
+        single = meta is not None and meta.decode_bucket is not None
+        if (not single and q.dtype == torch.bfloat16 and hq // hk <= 32
+                and self._query("jle_attention_mfma_supported", dh, hq, hk, ps)):
+            # portions of prompts in bfloat16: the matrix-core kernel, a wavefront per (tile of 32 tokens, head),
+            # which takes the kept keys before a tile's window as a range of its own; a step of single tokens
+            # goes on below (a query's keys shared between wavefronts)
+            seg_lens, _ = self._segments(meta, token_segment, positions)
+            if any(ln > 1 for ln in seg_lens):
+                tiles = meta.meta.get("kept_tiles") if meta is not None else None
+                if tiles is None:
+                    flat, o = [], 0
+                    for ln in seg_lens:
+                        for t in range(0, ln, self.PREFILL_TILE):
+                            flat += [o + t, min(self.PREFILL_TILE, ln - t)]
+                        o += ln
+                    tiles = torch.tensor(flat, dtype=torch.int32).to(q.device)
+                    if meta is not None:
+                        meta.meta["kept_tiles"] = tiles
+                self._call("jle_attention_prefill_kept", _p(q), _p(kv_cache), _p(out), _p(positions),
+                           _p(token_segment), _p(block_table), block_table.shape[1], _p(tiles), tiles.numel() // 2,
+                           self.PREFILL_TILE, param, keep, float(scale), hq, hk, dh, ps)
+                return out
         splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
         waves = n * hq
         if waves < self.GENERIC_SPLIT_BELOW:  # few tokens with many keys: a query's keys shared between wavefronts

@@ -250,6 +250,29 @@ def test_one_key_that_stands_out_at_the_windows_edges(folders, device, decoding,
     assert (moved > 1e-2) == (back not in ("first_not_kept", "just_outside")), moved
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("decoding", [False, True])
+@pytest.mark.parametrize("back", ["first", "last_kept", "first_not_kept", "just_outside", "just_inside", "page_edge"])
+def test_one_key_that_stands_out_on_the_matrix_core_kernels(folders_bf16, decoding, back):
+    """The same in bfloat16 at head sizes that the matrix-core attention kernels take (window 80, 5 tokens kept)."""
+    name, layer = "SF", 0
+    cfg, w = P.load(folders_bf16[name])
+    W, K = 80, 5
+    T = 290
+    special = {"first": 0, "last_kept": K - 1, "first_not_kept": K, "just_outside": T - 1 - W, "just_inside": T - W,
+               "page_edge": T - 1 - 63}[back]
+    x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(9)).bfloat16().float()
+    x[special] = 2.0 * x[T - 1]
+    want = _plain_mixer(cfg, w, layer, x, change=_sharpen_left_plain)
+    sizes = [special + 3] + [1] * (T - special - 3) if decoding else [T]
+    got = _mixer_alone(folders_bf16[name], "cuda:0", layer, sizes, x, dtype="bfloat16", change=_sharpen_left)
+    assert (got - want).abs().max() < 3e-2 * want.abs().max(), (got - want).abs().max() / want.abs().max()
+    x2 = x.clone()
+    x2[special] = torch.randn(cfg["width"], generator=torch.Generator().manual_seed(1))
+    moved = (_plain_mixer(cfg, w, layer, x2, change=_sharpen_left_plain)[T - 1] - want[T - 1]).abs().max()
+    assert (moved > 1e-1 * want.abs().max()) == (back not in ("first_not_kept", "just_outside")), moved
+
+
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("decoding", [False, True])
 def test_two_score_maps_with_sharp_scores_at_the_windows_edge(folders, device, decoding):
