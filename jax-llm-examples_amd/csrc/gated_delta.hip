@@ -22,7 +22,7 @@ __global__ __launch_bounds__(64) void gdr_prepare_kernel(const T* __restrict__ r
                                                          const float* __restrict__ dt_bias, float* __restrict__ qn,
                                                          float* __restrict__ kn, float* __restrict__ beta,
                                                          float* __restrict__ decay, float floor, int H, int G, int dk,
-                                                         int dv) {
+                                                         int dv, int dkp) {
   const int n = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
   const int C = 2 * G * dk + H * dv;
   if (g == G) {  // the write strengths and decays of the token's heads
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(64) void gdr_prepare_kernel(const T* __restrict__ r
   }
   for (int which = 0; which < 2; ++which) {
     const T* src = rows + (size_t)n * C + (size_t)(which * G + g) * dk;
-    float* dst = (which == 0 ? qn : kn) + ((size_t)n * G + g) * dk;
+    float* dst = (which == 0 ? qn : kn) + ((size_t)n * G + g) * dkp;  // (rows of dkp >= dk floats, zeros behind)
     float ss = 0.f;
     for (int e = lane; e < dk; e += 64) {
       const float x = Num<T>::load(src + e);
@@ -44,25 +44,39 @@ __global__ __launch_bounds__(64) void gdr_prepare_kernel(const T* __restrict__ r
     }
     float inv = 1.0f / sqrtf(wave_sum(ss) + floor);
     if (which == 0) inv *= 1.0f / sqrtf((float)dk);
-    for (int e = lane; e < dk; e += 64) dst[e] = Num<T>::load(src + e) * inv;
+    for (int e = lane; e < dkp; e += 64) dst[e] = e < dk ? Num<T>::load(src + e) * inv : 0.f;
   }
 }
 
-template <typename T, int R>
+// KS lanes share a column, each with R consecutive rows of it (KS * R = dkp >= dk, the unit vectors' rows padded with
+// zeros to that).  The wavefront brings the unit vectors, write strengths and decays of TB tokens into shared memory
+// at a time (asked for while the TB tokens before are worked on), and a lane its own values into registers.
+template <int KS, int R>
+struct ScanShape {
+  static constexpr int kDkp = KS * R;
+  static constexpr int kTB = kDkp <= 256 ? 16 : kDkp <= 512 ? 8 : kDkp <= 1024 ? 4 : 2;
+  static constexpr int kVecs = (kTB * kDkp / 4 + 63) / 64;  // 16-byte pieces a lane brings in per array
+};
+
+template <typename T, int KS, int R>
 __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows, const float* __restrict__ qn,
                                                       const float* __restrict__ kn, const float* __restrict__ beta,
                                                       const float* __restrict__ decay, float* __restrict__ state,
                                                       const int* __restrict__ cu_seqlens,
                                                       const int* __restrict__ state_slots,
                                                       const int* __restrict__ state_phase, float* __restrict__ o_raw,
-                                                      int H, int G, int dk, int dv, int KS) {
+                                                      int H, int G, int dk, int dv) {
+  using Shape = ScanShape<KS, R>;
+  constexpr int TB = Shape::kTB, DKP = Shape::kDkp, NV = Shape::kVecs, cols = 64 / KS;
+  __shared__ float4 sk[TB * DKP / 4], sq[TB * DKP / 4];
+  __shared__ float sb[TB], sg[TB];
   const int seg = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int cols = 64 / KS;
   const int ks = lane / cols, c = blockIdx.z * cols + (lane - ks * cols);
   const bool live = c < dv;
   const int g = h / (H / G);
   const int C = 2 * G * dk + H * dv;
   const int t0 = cu_seqlens[seg], t1 = cu_seqlens[seg + 1];
+  if (t0 >= t1) return;
   const size_t slot = (size_t)state_slots[seg];
   const int phase = state_phase[seg];
   const float* s_old = state + ((slot * 2 + phase) * H + h) * (size_t)dk * dv;
@@ -71,53 +85,85 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   float S[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) S[i] = (live && k0 + i < dk) ? s_old[(size_t)(k0 + i) * dv + c] : 0.f;
-  // this token's rows and the next one's, each in registers of its own (asked for a token ahead)
-  float kc[R], qc[R], vc = 0.f, bc = 0.f, gc = 1.f;
-  auto fetch = [&](int t, float (&k_)[R], float (&q_)[R], float& v_, float& b_, float& g_) {
-    const float* kp = kn + ((size_t)t * G + g) * dk + k0;
-    const float* qp = qn + ((size_t)t * G + g) * dk + k0;
+
+  float4 stk[NV], stq[NV];
+  float vnext[TB], vcur[TB], bnext = 0.f, gnext = 1.f;
+  auto ask = [&](int tb) {  // the TB tokens from tb on (those beyond the segment's end: its last token again, unused)
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      k_[i] = k0 + i < dk ? kp[i] : 0.f;
-      q_[i] = k0 + i < dk ? qp[i] : 0.f;
+    for (int j = 0; j < NV; ++j) {
+      const int f = lane + 64 * j;
+      if (f < TB * DKP / 4) {
+        const int tt = f / (DKP / 4), off = f - tt * (DKP / 4);
+        const size_t row = ((size_t)min(tb + tt, t1 - 1) * G + g) * DKP;
+        stk[j] = reinterpret_cast<const float4*>(kn + row)[off];
+        stq[j] = reinterpret_cast<const float4*>(qn + row)[off];
+      }
     }
-    v_ = live ? Num<T>::load(rows + (size_t)t * C + 2 * G * dk + (size_t)h * dv + c) : 0.f;
-    b_ = beta[(size_t)t * H + h];
-    g_ = decay[(size_t)t * H + h];
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt)
+      vnext[tt] = live ? Num<T>::load(rows + (size_t)min(tb + tt, t1 - 1) * C + 2 * G * dk + (size_t)h * dv + c) : 0.f;
+    if (lane < TB) {
+      const size_t at = (size_t)min(tb + lane, t1 - 1) * H + h;
+      bnext = beta[at];
+      gnext = decay[at];
+    }
   };
-  if (t0 < t1) fetch(t0, kc, qc, vc, bc, gc);
-  for (int t = t0; t < t1; ++t) {
-    float kx[R], qx[R], vx = 0.f, bx = 0.f, gx = 1.f;
-    if (t + 1 < t1) {
-      fetch(t + 1, kx, qx, vx, bx, gx);
-    } else {
+  auto put = [&]() {
 #pragma unroll
-      for (int i = 0; i < R; ++i) kx[i] = qx[i] = 0.f;
+    for (int j = 0; j < NV; ++j) {
+      const int f = lane + 64 * j;
+      if (f < TB * DKP / 4) {
+        sk[f] = stk[j];
+        sq[f] = stq[j];
+      }
     }
-    float dot = 0.f;
+    if (lane < TB) {
+      sb[lane] = bnext;
+      sg[lane] = gnext;
+    }
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      S[i] *= gc;
-      dot = __builtin_fmaf(S[i], kc[i], dot);
-    }
-    for (int o = cols; o < 64; o <<= 1) dot += __shfl_xor(dot, o, 64);
-    const float u = bc * (vc - dot);
-    float out = 0.f;
+    for (int tt = 0; tt < TB; ++tt) vcur[tt] = vnext[tt];
+  };
+  ask(t0);
+  put();
+  __syncthreads();
+  for (int tb = t0; tb < t1; tb += TB) {
+    const bool more = tb + TB < t1;
+    if (more) ask(tb + TB);
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      S[i] = __builtin_fmaf(kc[i], u, S[i]);
-      out = __builtin_fmaf(S[i], qc[i], out);
-    }
-    for (int o = cols; o < 64; o <<= 1) out += __shfl_xor(out, o, 64);
-    if (live && ks == 0) o_raw[((size_t)t * H + h) * dv + c] = out;
+    for (int tt = 0; tt < TB; ++tt) {
+      if (tb + tt < t1) {
+        float kc[R], qc[R];
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      kc[i] = kx[i];
-      qc[i] = qx[i];
+        for (int i = 0; i < R; i += 4) {
+          const float4 a = sk[(tt * DKP + k0 + i) / 4], b = sq[(tt * DKP + k0 + i) / 4];
+          kc[i] = a.x; kc[i + 1] = a.y; kc[i + 2] = a.z; kc[i + 3] = a.w;
+          qc[i] = b.x; qc[i + 1] = b.y; qc[i + 2] = b.z; qc[i + 3] = b.w;
+        }
+        const float gc = sg[tt], bc = sb[tt];
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+          S[i] *= gc;
+          dot = __builtin_fmaf(S[i], kc[i], dot);
+        }
+#pragma unroll
+        for (int o = cols; o < 64; o <<= 1) dot += __shfl_xor(dot, o, 64);
+        const float u = bc * (vcur[tt] - dot);
+        float out = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+          S[i] = __builtin_fmaf(kc[i], u, S[i]);
+          out = __builtin_fmaf(S[i], qc[i], out);
+        }
+#pragma unroll
+        for (int o = cols; o < 64; o <<= 1) out += __shfl_xor(out, o, 64);
+        if (live && ks == 0) o_raw[((size_t)(tb + tt) * H + h) * dv + c] = out;
+      }
     }
-    vc = vx;
-    bc = bx;
-    gc = gx;
+    __syncthreads();
+    if (more) put();
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -148,22 +194,30 @@ template <typename T>
 int launch_gdr(const T* rows, const float* gates, const float* a_log, const float* dt_bias, const float* norm_w,
                const T* gate, float* state, const int* cu_seqlens, const int* state_slots, const int* state_phase,
                float* qn, float* kn, float* beta, float* decay, float* o_raw, T* out, int N, int R_, int H, int G, int dk,
-               int dv, float eps, float floor, hipStream_t s) {
-  hipLaunchKernelGGL(gdr_prepare_kernel<T>, dim3(N, G + 1), dim3(64), 0, s, rows, gates, a_log, dt_bias, qn, kn, beta,
-                     decay, floor, H, G, dk, dv);
-  JLE_LAUNCH_CHECK();
+               int dv, int dkp, float eps, float floor, hipStream_t s) {
   // lanes a column: the fewest that leave a lane at most 16 rows of it (by the sizes alone)
   int KS = 1;
   while (KS < 64 && (dk + KS - 1) / KS > 16) KS <<= 1;
   const int per = (dk + KS - 1) / KS, cols = 64 / KS;
+  const int RR = per <= 4 ? 4 : per <= 8 ? 8 : per <= 16 ? 16 : 32;
+  if (dkp != KS * RR) return JLE_BAD_ARG;
+  hipLaunchKernelGGL(gdr_prepare_kernel<T>, dim3(N, G + 1), dim3(64), 0, s, rows, gates, a_log, dt_bias, qn, kn, beta,
+                     decay, floor, H, G, dk, dv, dkp);
+  JLE_LAUNCH_CHECK();
   const dim3 grid(R_, H, (dv + cols - 1) / cols);
-#define JLE_SCAN(RR)                                                                                               \
-  hipLaunchKernelGGL((gdr_scan_kernel<T, RR>), grid, dim3(64), 0, s, rows, qn, kn, beta, decay, state, cu_seqlens, \
-                     state_slots, state_phase, o_raw, H, G, dk, dv, KS)
-  if (per <= 4) JLE_SCAN(4);
-  else if (per <= 8) JLE_SCAN(8);
-  else if (per <= 16) JLE_SCAN(16);
-  else JLE_SCAN(32);
+#define JLE_SCAN(KS_, RR_)                                                                                          \
+  hipLaunchKernelGGL((gdr_scan_kernel<T, KS_, RR_>), grid, dim3(64), 0, s, rows, qn, kn, beta, decay, state, cu_seqlens, \
+                     state_slots, state_phase, o_raw, H, G, dk, dv)
+  if (KS == 1 && RR == 4) JLE_SCAN(1, 4);
+  else if (KS == 1 && RR == 8) JLE_SCAN(1, 8);
+  else if (KS == 1) JLE_SCAN(1, 16);
+  else if (KS == 2) JLE_SCAN(2, 16);
+  else if (KS == 4) JLE_SCAN(4, 16);
+  else if (KS == 8) JLE_SCAN(8, 16);
+  else if (KS == 16) JLE_SCAN(16, 16);
+  else if (KS == 32) JLE_SCAN(32, 16);
+  else if (RR <= 16) JLE_SCAN(64, 16);
+  else JLE_SCAN(64, 32);
 #undef JLE_SCAN
   JLE_LAUNCH_CHECK();
   hipLaunchKernelGGL(gdr_out_kernel<T>, dim3(N, H), dim3(64), 0, s, o_raw, gate, norm_w, out, eps, H, dv);
@@ -173,23 +227,35 @@ int launch_gdr(const T* rows, const float* gates, const float* a_log, const floa
 
 }  // namespace
 
+// The width of a unit vector's row in the scratch arrays: dk rounded up to lanes a column x rows a lane.
+JLE_API int jle_gated_delta_padded(int dk) {
+  if (dk <= 0 || dk > 2048) return -1;
+  int KS = 1;
+  while (KS < 64 && (dk + KS - 1) / KS > 16) KS <<= 1;
+  const int per = (dk + KS - 1) / KS;
+  return KS * (per <= 4 ? 4 : per <= 8 ? 8 : per <= 16 ? 16 : 32);
+}
+
 // rows [N, 2 G dk + H dv] (q | k | v behind convolution and activation) and gate [N, H dv] in the run dtype; gates
 // float32 [N, 2 H] (write strengths, then decays, before their biases and squashing); state float32 [slots, 2, H, dk,
-// dv]; qn, kn [N, G, dk], beta, decay [N, H], o_raw [N, H, dv]: float32 scratch; out [N, H dv] in the run dtype.
+// dv]; qn, kn [N, G, dkp] (dkp = jle_gated_delta_padded(dk), 16-byte aligned), beta, decay [N, H], o_raw [N, H, dv]:
+// float32 scratch; out [N, H dv] in the run dtype.
 JLE_API int jle_gated_delta(const void* rows, int is_bf16, const float* gates, const float* a_log, const float* dt_bias,
                             const float* norm_w, const void* gate, float* state, const int* cu_seqlens,
                             const int* state_slots, const int* state_phase, float* qn, float* kn, float* beta,
                             float* decay, float* o_raw, void* out, int N, int R, int H, int G, int dk, int dv, float eps,
                             float floor, hipStream_t s) {
   if (N <= 0) return 0;
+  const int dkp = jle_gated_delta_padded(dk);
+  if (dkp <= 0 || ((uintptr_t)qn | (uintptr_t)kn) % 16) return JLE_BAD_ARG;
   if (R <= 0 || H <= 0 || G <= 0 || H % G || dk <= 0 || dk > 2048 || dv <= 0 || H > 65535 || G + 1 > 65535 ||
       rows == nullptr || gates == nullptr || state == nullptr || out == nullptr || gate == nullptr)
     return JLE_BAD_ARG;
   if (is_bf16)
     return launch_gdr<bf16_t>((const bf16_t*)rows, gates, a_log, dt_bias, norm_w, (const bf16_t*)gate, state, cu_seqlens,
-                              state_slots, state_phase, qn, kn, beta, decay, o_raw, (bf16_t*)out, N, R, H, G, dk, dv, eps,
-                              floor, s);
+                              state_slots, state_phase, qn, kn, beta, decay, o_raw, (bf16_t*)out, N, R, H, G, dk, dv, dkp,
+                              eps, floor, s);
   return launch_gdr<float>((const float*)rows, gates, a_log, dt_bias, norm_w, (const float*)gate, state, cu_seqlens,
-                           state_slots, state_phase, qn, kn, beta, decay, o_raw, (float*)out, N, R, H, G, dk, dv, eps,
+                           state_slots, state_phase, qn, kn, beta, decay, o_raw, (float*)out, N, R, H, G, dk, dv, dkp, eps,
                            floor, s);
 }

@@ -163,7 +163,8 @@ def _bind(path: str):
     for name, args in (("jle_attention_mfma_supported", [_i, _i, _i, _i]),  # queries, not launches: no stream
                        ("jle_gemm_stream_supported", [_i, _i, _i]), ("jle_gemm_f32_stream_supported", [_i, _i, _i]),
                        ("jle_latent_attention_mfma_supported", [_i, _i, _i, _i, _i]), ("jle_attention_group_waves", []),
-                       ("jle_mlstm_chunked_supported", [_i, _i]), ("jle_mlstm_chunk_tokens", [])):
+                       ("jle_mlstm_chunked_supported", [_i, _i]), ("jle_mlstm_chunk_tokens", []),
+                       ("jle_gated_delta_padded", [_i])):
         fn = getattr(lib, name, None)
         if fn is not None:
             fn.argtypes = args
@@ -911,9 +912,12 @@ class HipOps:
                                (ctx.state_phase, "state phases", (ctx.num_segments,))):
             self._chk(t, torch.int32, shape, what)
         dev = rows.device
-        scratch = torch.empty(n * (2 * G * dk + 2 * H + H * dv), dtype=torch.float32, device=dev)
-        qn, kn = scratch[: n * G * dk], scratch[n * G * dk: 2 * n * G * dk]
-        o = 2 * n * G * dk
+        dkp = self._query("jle_gated_delta_padded", dk)  # (the unit vectors' rows, filled up to what the scan's lanes hold)
+        if dkp < dk:
+            raise KernelError(f"the gated delta rule's kernels take keys of up to 2048 elements, not {dk}")
+        scratch = torch.empty(n * (2 * G * dkp + 2 * H + H * dv), dtype=torch.float32, device=dev)
+        qn, kn = scratch[: n * G * dkp], scratch[n * G * dkp: 2 * n * G * dkp]
+        o = 2 * n * G * dkp
         beta, decay, o_raw = scratch[o: o + n * H], scratch[o + n * H: o + 2 * n * H], scratch[o + 2 * n * H:]
         out = torch.empty(n, H * dv, dtype=rows.dtype, device=dev)
         self._call("jle_gated_delta", _p(rows), self._is_bf16(rows), _p(gates), _p(a_log), _p(dt_bias), _p(norm_weight),
