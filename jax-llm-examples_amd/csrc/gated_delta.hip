@@ -4,9 +4,9 @@
 // g = exp(-exp(A) softplus(a + dt)).  Three kernels:
 //   gdr_prepare_kernel   the unit vectors (float32), beta and the decay of every token of the step
 //   gdr_scan_kernel      the recurrence: a column of S depends on nothing but itself, k, q, v of its own place, beta
-//                        and g, so a wavefront takes 64 / KS columns of one head, KS lanes share a column (each
-//                        holds R consecutive rows of it in registers), and the two dot products are finished with
-//                        KS - 1 lane swaps; the next token's rows are asked for before this token's are used
+//                        and g, so a wavefront takes 64 / KS columns of one head, KS neighbouring lanes share a
+//                        column (each holds R consecutive rows of it in registers), and the two dot products are
+//                        finished with log2(KS) lane swaps; the next tokens' rows are asked for before these are used
 //   gdr_out_kernel       o / sqrt(mean(o^2) + eps) * w * silu(gate), rounded to the run dtype
 // The memory lies [slot][half][H][dk][dv]; a step reads the half `phase` and writes the other.  Every sum is formed
 // in an order that depends on the sizes alone, token after token: cutting a sequence into steps changes no bit.
@@ -51,6 +51,23 @@ __global__ __launch_bounds__(64) void gdr_prepare_kernel(const T* __restrict__ r
 // KS lanes share a column, each with R consecutive rows of it (KS * R = dkp >= dk, the unit vectors' rows padded with
 // zeros to that).  The wavefront brings the unit vectors, write strengths and decays of TB tokens into shared memory
 // at a time (asked for while the TB tokens before are worked on), and a lane its own values into registers.
+// the sum over the KS neighbouring lanes that share a column (every one of them gets it, the same bits in all):
+// within a row of 16 lanes by the lane-permuting operand modes, beyond by the cross-lane read
+template <int CTRL>
+__device__ __forceinline__ float lanes_permuted(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int KS>
+__device__ __forceinline__ float column_lanes_sum(float v) {
+  if (KS >= 2) v += lanes_permuted<0xB1>(v);    // lanes 1 0 3 2 of every four
+  if (KS >= 4) v += lanes_permuted<0x4E>(v);    // lanes 2 3 0 1 of every four
+  if (KS >= 8) v += lanes_permuted<0x141>(v);   // every eight mirrored
+  if (KS >= 16) v += lanes_permuted<0x140>(v);  // every sixteen mirrored
+  if (KS >= 32) v += __shfl_xor(v, 16, 64);
+  if (KS >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
 template <int KS, int R>
 struct ScanShape {
   static constexpr int kDkp = KS * R;
@@ -71,7 +88,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   __shared__ float4 sk[TB * DKP / 4], sq[TB * DKP / 4];
   __shared__ float sb[TB], sg[TB];
   const int seg = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int ks = lane / cols, c = blockIdx.z * cols + (lane - ks * cols);
+  const int ks = lane % KS, c = blockIdx.z * cols + lane / KS;  // (a column's lanes are neighbours)
   const bool live = c < dv;
   const int g = h / (H / G);
   const int C = 2 * G * dk + H * dv;
@@ -141,23 +158,21 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
           qc[i] = b.x; qc[i + 1] = b.y; qc[i + 2] = b.z; qc[i + 3] = b.w;
         }
         const float gc = sg[tt], bc = sb[tt];
-        float dot = 0.f;
+        float d4[4] = {0.f, 0.f, 0.f, 0.f};  // (four sums side by side: no chain of R dependent operations)
 #pragma unroll
         for (int i = 0; i < R; ++i) {
           S[i] *= gc;
-          dot = __builtin_fmaf(S[i], kc[i], dot);
+          d4[i & 3] = __builtin_fmaf(S[i], kc[i], d4[i & 3]);
         }
-#pragma unroll
-        for (int o = cols; o < 64; o <<= 1) dot += __shfl_xor(dot, o, 64);
+        const float dot = column_lanes_sum<KS>((d4[0] + d4[1]) + (d4[2] + d4[3]));
         const float u = bc * (vcur[tt] - dot);
-        float out = 0.f;
+        float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < R; ++i) {
           S[i] = __builtin_fmaf(kc[i], u, S[i]);
-          out = __builtin_fmaf(S[i], qc[i], out);
+          o4[i & 3] = __builtin_fmaf(S[i], qc[i], o4[i & 3]);
         }
-#pragma unroll
-        for (int o = cols; o < 64; o <<= 1) out += __shfl_xor(out, o, 64);
+        const float out = column_lanes_sum<KS>((o4[0] + o4[1]) + (o4[2] + o4[3]));
         if (live && ks == 0) o_raw[((size_t)(tb + tt) * H + h) * dv + c] = out;
       }
     }

@@ -552,6 +552,13 @@ JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates
   return 0;
 }
 
+// The logits alone (for a choice that another kernel makes).
+JLE_API int jle_moe_logits(const float* h, const float* w, float* logits, int N, int D, int E, hipStream_t s) {
+  if (N <= 0) return 0;
+  if (E < 1 || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
+  return launch_logits(h, w, logits, N, D, E, s);
+}
+
 // The router and the grouping of its choices in one call (the same results as jle_moe_route, then jle_moe_align).
 // extra_group: offsets has E + 2 entries, sorted_token and sorted_gate N * k + N (see align_by_block).
 JLE_API int jle_moe_route_align(const float* h, const float* w, int* ids, float* gates, float* logits, int* offsets,

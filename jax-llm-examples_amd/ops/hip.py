@@ -88,7 +88,8 @@ _SIGNATURES = {
                           _i, _i, _f, _f, _f, _vp],
     "jle_span_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_row_gate": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
-    "jle_scaled_add_norm": [_vp, _vp, _i, _f, _vp, _i, _f, _vp, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
+    "jle_scaled_add_norm": [_vp, _vp, _i, _f, _vp, _i, _f, _vp, _vp, _f, _vp, _i, _vp, _i, _i, _vp, _i, _vp],
+    "jle_moe_logits": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_heads_prepare": [_vp, _vp, _vp, _vp, _i, _i, _f, _f, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i,
                           _vp],
     "jle_diff_combine": [_vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _vp],
@@ -644,8 +645,16 @@ class HipOps:
         sqrt(mean(x^2) + eps) * weight`` in the run dtype and, if wanted, float32; one launch."""
         n, d = x.shape
         self._chk(x, torch.float32, (n, d), "residual")
-        terms = [(self.materialize(t), f) for t, f in delta.terms]
-        for t, _ in terms:
+        terms = list(delta.terms)
+        inv, inv_k = None, 0
+        if isinstance(terms[0][0], ExpertSum) and terms[0][0].shared is None:  # (its pieces are added up by the kernel)
+            pieces = terms[0][0]
+            inv, inv_k = pieces.inv, pieces.k
+            terms[0] = (pieces.routed, terms[0][1])
+            self._chk(pieces.routed, None, (pieces.routed.shape[0], d), "expert outputs")
+            self._chk(inv, torch.int32, (n * inv_k,), "rows of the expert outputs")
+        terms = [(self.materialize(t), f) for t, f in terms]
+        for t, _ in terms[(1 if inv is not None else 0):]:
             self._chk(t, None, (n, d), "branch output")
         kind = lambda t: 1 if t.dtype == torch.bfloat16 else 2 if t.dtype == torch.float32 else self._is_bf16(t)
         (a, fa), (b, fb) = terms[0], (terms[1] if len(terms) > 1 else (None, 0.0))
@@ -657,7 +666,7 @@ class HipOps:
         h32 = torch.empty(n, d, dtype=torch.float32, device=x.device) if norm and want32 else None
         self._call("jle_scaled_add_norm", _p(x), _p(a), kind(a), float(fa), _p(b), 0 if b is None else kind(b),
                    float(fb), _p(delta.vector), _p(weight), float(eps), _p(h),
-                   1 if out_dtype == torch.bfloat16 else 0, _p(h32), n, d)
+                   1 if out_dtype == torch.bfloat16 else 0, _p(h32), n, d, _p(inv), inv_k)
         return h, h32
 
     def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):
@@ -1605,10 +1614,8 @@ class HipOps:
         if correction is not None:
             self._chk(correction, torch.float32, (e,), "correction")
         dev = h32.device
-        ids1 = torch.empty(n, 1, dtype=torch.int32, device=dev)
-        gates1 = torch.empty(n, 1, dtype=torch.float32, device=dev)
         logits = torch.empty(n, e, dtype=torch.float32, device=dev)
-        self._call("jle_moe_route", _p(h32), _p(router), _p(ids1), _p(gates1), _p(logits), n, d, e, 1)
+        self._call("jle_moe_logits", _p(h32), _p(router), _p(logits), n, d, e)
         ids = torch.empty(n, top_k, dtype=torch.int32, device=dev)
         weights = torch.empty(n, top_k, dtype=torch.float32, device=dev)
         self._call("jle_moe_choose", _p(logits), _p(correction), _p(ids), _p(weights), n, e, top_k,
