@@ -8,7 +8,7 @@
 //                        column (each holds R consecutive rows of it in registers), and the two dot products are
 //                        finished with log2(KS) lane swaps; the next tokens' rows are asked for before these are used
 //   gdr_out_kernel       o / sqrt(mean(o^2) + eps) * w * silu(gate), rounded to the run dtype
-// The memory lies [slot][half][H][dk][dv]; a step reads the half `phase` and writes the other.  Every sum is formed
+// The memory lies [slot][half][H][dv][dk] (a column's rows together); a step reads the half `phase` and writes the other.  Every sum is formed
 // in an order that depends on the sizes alone, token after token: cutting a sequence into steps changes no bit.
 #include "common.h"
 
@@ -68,6 +68,8 @@ __device__ __forceinline__ float column_lanes_sum(float v) {
   return v;
 }
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));  // (a plain vector type: arrays of it stay in registers)
+
 template <int KS, int R>
 struct ScanShape {
   static constexpr int kDkp = KS * R;
@@ -85,7 +87,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
                                                       int H, int G, int dk, int dv) {
   using Shape = ScanShape<KS, R>;
   constexpr int TB = Shape::kTB, DKP = Shape::kDkp, NV = Shape::kVecs, cols = 64 / KS;
-  __shared__ float4 sk[TB * DKP / 4], sq[TB * DKP / 4];
+  __shared__ f32x4 sk[TB * DKP / 4], sq[TB * DKP / 4];
   __shared__ float sb[TB], sg[TB];
   const int seg = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int ks = lane % KS, c = blockIdx.z * cols + lane / KS;  // (a column's lanes are neighbours)
@@ -101,31 +103,49 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   const int k0 = ks * R;
   float S[R];
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = (live && k0 + i < dk) ? s_old[(size_t)(k0 + i) * dv + c] : 0.f;
+  for (int i = 0; i < R; ++i) S[i] = 0.f;
+  // (a column's dk rows lie together: its KS lanes read neighbouring pieces of R floats)
+  if (live) {
+    if (dk % 4 == 0) {
+#pragma unroll
+      for (int i = 0; i < R; i += 4) {
+        if (k0 + i < dk) {
+          const float4 v = *reinterpret_cast<const float4*>(s_old + (size_t)c * dk + k0 + i);
+          S[i] = v.x; S[i + 1] = v.y; S[i + 2] = v.z; S[i + 3] = v.w;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        if (k0 + i < dk) S[i] = s_old[(size_t)c * dk + k0 + i];
+    }
+  }
 
-  float4 stk[NV], stq[NV];
+  f32x4 stk[NV], stq[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) stk[j] = stq[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   float vnext[TB], vcur[TB], bnext = 0.f, gnext = 1.f;
-  auto ask = [&](int tb) {  // the TB tokens from tb on (those beyond the segment's end: its last token again, unused)
+  auto ask = [&](int tb) __attribute__((always_inline)) {  // the TB tokens from tb on (those beyond the segment's end: its last token again, unused)
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int f = lane + 64 * j;
       if (f < TB * DKP / 4) {
         const int tt = f / (DKP / 4), off = f - tt * (DKP / 4);
         const size_t row = ((size_t)min(tb + tt, t1 - 1) * G + g) * DKP;
-        stk[j] = reinterpret_cast<const float4*>(kn + row)[off];
-        stq[j] = reinterpret_cast<const float4*>(qn + row)[off];
+        stk[j] = reinterpret_cast<const f32x4*>(kn + row)[off];
+        stq[j] = reinterpret_cast<const f32x4*>(qn + row)[off];
       }
     }
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt)
       vnext[tt] = live ? Num<T>::load(rows + (size_t)min(tb + tt, t1 - 1) * C + 2 * G * dk + (size_t)h * dv + c) : 0.f;
-    if (lane < TB) {
+    if (lane < TB) {  // (places behind the segment's end: a step that changes nothing, no write and no decay)
       const size_t at = (size_t)min(tb + lane, t1 - 1) * H + h;
-      bnext = beta[at];
-      gnext = decay[at];
+      bnext = tb + lane < t1 ? beta[at] : 0.f;
+      gnext = tb + lane < t1 ? decay[at] : 1.f;
     }
   };
-  auto put = [&]() {
+  auto put = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int f = lane + 64 * j;
@@ -147,43 +167,55 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   for (int tb = t0; tb < t1; tb += TB) {
     const bool more = tb + TB < t1;
     if (more) ask(tb + TB);
+    auto token = [&](int tt) __attribute__((always_inline)) {
+      float kc[R], qc[R];
 #pragma unroll
-    for (int tt = 0; tt < TB; ++tt) {
-      if (tb + tt < t1) {
-        float kc[R], qc[R];
-#pragma unroll
-        for (int i = 0; i < R; i += 4) {
-          const float4 a = sk[(tt * DKP + k0 + i) / 4], b = sq[(tt * DKP + k0 + i) / 4];
-          kc[i] = a.x; kc[i + 1] = a.y; kc[i + 2] = a.z; kc[i + 3] = a.w;
-          qc[i] = b.x; qc[i + 1] = b.y; qc[i + 2] = b.z; qc[i + 3] = b.w;
-        }
-        const float gc = sg[tt], bc = sb[tt];
-        float d4[4] = {0.f, 0.f, 0.f, 0.f};  // (four sums side by side: no chain of R dependent operations)
-#pragma unroll
-        for (int i = 0; i < R; ++i) {
-          S[i] *= gc;
-          d4[i & 3] = __builtin_fmaf(S[i], kc[i], d4[i & 3]);
-        }
-        const float dot = column_lanes_sum<KS>((d4[0] + d4[1]) + (d4[2] + d4[3]));
-        const float u = bc * (vcur[tt] - dot);
-        float o4[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int i = 0; i < R; ++i) {
-          S[i] = __builtin_fmaf(kc[i], u, S[i]);
-          o4[i & 3] = __builtin_fmaf(S[i], qc[i], o4[i & 3]);
-        }
-        const float out = column_lanes_sum<KS>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-        if (live && ks == 0) o_raw[((size_t)(tb + tt) * H + h) * dv + c] = out;
+      for (int i = 0; i < R; i += 4) {
+        const f32x4 a = sk[(tt * DKP + k0 + i) / 4], b = sq[(tt * DKP + k0 + i) / 4];
+        kc[i] = a.x; kc[i + 1] = a.y; kc[i + 2] = a.z; kc[i + 3] = a.w;
+        qc[i] = b.x; qc[i + 1] = b.y; qc[i + 2] = b.z; qc[i + 3] = b.w;
       }
+      const float gc = sg[tt], bc = sb[tt];
+      float d4[4] = {0.f, 0.f, 0.f, 0.f};  // (four sums side by side: no chain of R dependent operations)
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        S[i] *= gc;
+        d4[i & 3] = __builtin_fmaf(S[i], kc[i], d4[i & 3]);
+      }
+      const float dot = column_lanes_sum<KS>((d4[0] + d4[1]) + (d4[2] + d4[3]));
+      const float u = bc * (vcur[tt] - dot);
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        S[i] = __builtin_fmaf(kc[i], u, S[i]);
+        o4[i & 3] = __builtin_fmaf(S[i], qc[i], o4[i & 3]);
+      }
+      const float out = column_lanes_sum<KS>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+      if (live && ks == 0 && tb + tt < t1) o_raw[((size_t)(tb + tt) * H + h) * dv + c] = out;
+    };
+    if (tb + TB <= t1) {  // a whole block: no branch around a token, one stretch of code that the compiler may interleave
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt) token(tt);
+    } else {  // (the segment's last tokens, or all of a short one: no work for places behind its end)
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt)
+        if (tb + tt < t1) token(tt);
     }
     __syncthreads();
     if (more) put();
     __syncthreads();
   }
   if (live) {
+    if (dk % 4 == 0) {
 #pragma unroll
-    for (int i = 0; i < R; ++i)
-      if (k0 + i < dk) s_new[(size_t)(k0 + i) * dv + c] = S[i];
+      for (int i = 0; i < R; i += 4)
+        if (k0 + i < dk)
+          *reinterpret_cast<float4*>(s_new + (size_t)c * dk + k0 + i) = float4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        if (k0 + i < dk) s_new[(size_t)c * dk + k0 + i] = S[i];
+    }
   }
 }
 
@@ -213,26 +245,41 @@ int launch_gdr(const T* rows, const float* gates, const float* a_log, const floa
   // lanes a column: the fewest that leave a lane at most 16 rows of it (by the sizes alone)
   int KS = 1;
   while (KS < 64 && (dk + KS - 1) / KS > 16) KS <<= 1;
-  const int per = (dk + KS - 1) / KS, cols = 64 / KS;
+  const int per = (dk + KS - 1) / KS;
   const int RR = per <= 4 ? 4 : per <= 8 ? 8 : per <= 16 ? 16 : 32;
   if (dkp != KS * RR) return JLE_BAD_ARG;
   hipLaunchKernelGGL(gdr_prepare_kernel<T>, dim3(N, G + 1), dim3(64), 0, s, rows, gates, a_log, dt_bias, qn, kn, beta,
                      decay, floor, H, G, dk, dv, dkp);
   JLE_LAUNCH_CHECK();
-  const dim3 grid(R_, H, (dv + cols - 1) / cols);
+  // A step with few (segment, head) pairs leaves most of the machine idle, and what a token takes is the length of its
+  // chain of dependent operations: then a column gets more lanes with fewer rows each (the row's width stays).
+  int ks = KS, rr = RR;
+  while (rr > 4 && ks < 16 && (long long)R_ * H * ((dv + 64 / ks - 1) / (64 / ks)) < 1024) {  // (up to a row of 16 lanes)
+    ks <<= 1;
+    rr >>= 1;
+  }
+  const int cols_ = 64 / ks;
+  const dim3 grid(R_, H, (dv + cols_ - 1) / cols_);
 #define JLE_SCAN(KS_, RR_)                                                                                          \
   hipLaunchKernelGGL((gdr_scan_kernel<T, KS_, RR_>), grid, dim3(64), 0, s, rows, qn, kn, beta, decay, state, cu_seqlens, \
                      state_slots, state_phase, o_raw, H, G, dk, dv)
-  if (KS == 1 && RR == 4) JLE_SCAN(1, 4);
-  else if (KS == 1 && RR == 8) JLE_SCAN(1, 8);
-  else if (KS == 1) JLE_SCAN(1, 16);
-  else if (KS == 2) JLE_SCAN(2, 16);
-  else if (KS == 4) JLE_SCAN(4, 16);
-  else if (KS == 8) JLE_SCAN(8, 16);
-  else if (KS == 16) JLE_SCAN(16, 16);
-  else if (KS == 32) JLE_SCAN(32, 16);
-  else if (RR <= 16) JLE_SCAN(64, 16);
-  else JLE_SCAN(64, 32);
+#define JLE_SCAN_R(KS_)              \
+  do {                               \
+    if (rr == 4) JLE_SCAN(KS_, 4);   \
+    else if (rr == 8) JLE_SCAN(KS_, 8); \
+    else if (rr == 16) JLE_SCAN(KS_, 16); \
+    else JLE_SCAN(KS_, 32);          \
+  } while (0)
+  switch (ks) {
+    case 1: JLE_SCAN_R(1); break;
+    case 2: JLE_SCAN_R(2); break;
+    case 4: JLE_SCAN_R(4); break;
+    case 8: JLE_SCAN_R(8); break;
+    case 16: JLE_SCAN_R(16); break;
+    case 32: JLE_SCAN_R(32); break;
+    default: JLE_SCAN_R(64); break;
+  }
+#undef JLE_SCAN_R
 #undef JLE_SCAN
   JLE_LAUNCH_CHECK();
   hipLaunchKernelGGL(gdr_out_kernel<T>, dim3(N, H), dim3(64), 0, s, o_raw, gate, norm_w, out, eps, H, dv);
@@ -252,8 +299,8 @@ JLE_API int jle_gated_delta_padded(int dk) {
 }
 
 // rows [N, 2 G dk + H dv] (q | k | v behind convolution and activation) and gate [N, H dv] in the run dtype; gates
-// float32 [N, 2 H] (write strengths, then decays, before their biases and squashing); state float32 [slots, 2, H, dk,
-// dv]; qn, kn [N, G, dkp] (dkp = jle_gated_delta_padded(dk), 16-byte aligned), beta, decay [N, H], o_raw [N, H, dv]:
+// float32 [N, 2 H] (write strengths, then decays, before their biases and squashing); state float32 [slots, 2, H, dv,
+// dk]; qn, kn [N, G, dkp] (dkp = jle_gated_delta_padded(dk), 16-byte aligned), beta, decay [N, H], o_raw [N, H, dv]:
 // float32 scratch; out [N, H dv] in the run dtype.
 JLE_API int jle_gated_delta(const void* rows, int is_bf16, const float* gates, const float* a_log, const float* dt_bias,
                             const float* norm_w, const void* gate, float* state, const int* cu_seqlens,

@@ -913,7 +913,7 @@ class HipOps:
         self._chk(rows, None, (n, 2 * G * dk + H * dv), "q | k | v rows")
         self._chk(out_gate, rows.dtype, (n, H * dv), "output gate")
         self._chk(gates, torch.float32, (n, 2 * H), "gate pre-activations")
-        self._chk(state, torch.float32, (state.shape[0], 2, H, dk, dv), "memory")
+        self._chk(state, torch.float32, (state.shape[0], 2, H, dv, dk), "memory")
         for t, shape, what in ((a_log, (H,), "a_log"), (dt_bias, (H,), "dt_bias"), (norm_weight, (dv,), "head norm weight")):
             self._chk(t, torch.float32, shape, what)
         for t, what, shape in ((ctx.cu_seqlens, "segment bounds", (ctx.num_segments + 1,)),

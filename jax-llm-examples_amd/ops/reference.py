@@ -380,7 +380,7 @@ class ReferenceOps:
         float32 ``[N, 2 H]`` = the write strengths' and the decays' pre-activations.  Per kv head q and k become unit
         vectors (``x / sqrt(sum(x^2) + floor)``), q times ``dk^(-1/2)``; ``beta = sigmoid(.)``, ``g = exp(-exp(a_log)
         softplus(. + dt_bias))``; per head, token by token from the request's memory (``state[slot, phase]``: ``[H,
-        dk, dv]``; the new one goes to ``state[slot, 1 - phase]``): ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
+        dv, dk]``, the transposed ``S``; the new one goes to ``state[slot, 1 - phase]``): ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
         o = S^T q``.  Then ``o`` divided by its root mean square per head (``eps``), times ``norm_weight`` (``[dv]``),
         times ``silu(out_gate)``.  ``[N, H dv]`` in the run dtype."""
         n = rows.shape[0]
@@ -398,13 +398,13 @@ class ReferenceOps:
         cu = ctx.cu_seqlens.tolist()
         slots, phase = ctx.state_slots.tolist(), ctx.state_phase.tolist()
         for s in range(len(cu) - 1):
-            S = state[slots[s], phase[s]].float().clone()
+            S = state[slots[s], phase[s]].float().transpose(-1, -2).clone()
             for t in range(cu[s], cu[s + 1]):
                 S = decay[t][:, None, None] * S
                 u = beta[t][:, None] * (v[t] - torch.einsum("hkv,hk->hv", S, k[t]))
                 S = S + k[t][:, :, None] * u[:, None, :]
                 out[t] = torch.einsum("hkv,hk->hv", S, q[t])
-            state[slots[s], 1 - phase[s]] = S.to(state.dtype)
+            state[slots[s], 1 - phase[s]] = S.transpose(-1, -2).to(state.dtype)
         o = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
         g = out_gate.float()
         return (o.reshape(n, H * dv) * (g * torch.sigmoid(g))).to(rows.dtype)

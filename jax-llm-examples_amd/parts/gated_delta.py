@@ -70,7 +70,7 @@ class GatedDelta(Mixer):
         self.conv_by_tap = self.params["conv"].t().contiguous() if self.conv_taps else None
 
     def cache_need(self) -> CacheNeed:
-        states = [("memory", (2, self.num_heads, self.head_dim, self.value_dim), torch.float32)]
+        states = [("memory", (2, self.num_heads, self.value_dim, self.head_dim), torch.float32)]  # (S transposed)
         if self.conv_taps > 1:
             states.append(("conv", (2, self.conv_taps - 1, self.channels), self.state_dtype))
         return CacheNeed(states=tuple(states))
