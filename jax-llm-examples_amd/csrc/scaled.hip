@@ -30,11 +30,33 @@ __device__ __forceinline__ float term(const void* p, int is_bf16, size_t i) {
   return is_bf16 ? bf16_to_float(((const bf16_t*)p)[i]) : ((const float*)p)[i];
 }
 
-__device__ __forceinline__ float updated(const ScaledArgs& p, size_t base, int d) {
+constexpr int kPiecesInRegisters = 8;
+
+// where the pieces of row n's expert sum lie, looked up once per row (up to kPiecesInRegisters of them)
+struct Pieces {
+  size_t at[kPiecesInRegisters];
+  int count;  // -1: a is a plain row (or has more pieces than are kept here: looked up per element)
+};
+
+__device__ __forceinline__ Pieces pieces_of(const ScaledArgs& p, size_t n) {
+  Pieces r;
+  r.count = (p.a_inv != nullptr && p.a_k <= kPiecesInRegisters) ? p.a_k : -1;
+#pragma unroll
+  for (int j = 0; j < kPiecesInRegisters; ++j)
+    r.at[j] = j < r.count ? (size_t)p.a_inv[n * p.a_k + j] * p.D : 0;
+  return r;
+}
+
+__device__ __forceinline__ float updated(const ScaledArgs& p, const Pieces& pc, size_t base, int d) {
   float v = p.x[base + d];
   if (p.a != nullptr) {
     float ta;
-    if (p.a_inv != nullptr) {
+    if (pc.count >= 0) {
+      ta = 0.f;
+#pragma unroll
+      for (int j = 0; j < kPiecesInRegisters; ++j)
+        if (j < pc.count) ta += term(p.a, p.a_bf16, pc.at[j] + d);
+    } else if (p.a_inv != nullptr) {
       ta = 0.f;
       const int* rows = p.a_inv + (size_t)blockIdx.x * p.a_k;
       for (int j = 0; j < p.a_k; ++j) ta += term(p.a, p.a_bf16, (size_t)rows[j] * p.D + d);
@@ -54,18 +76,65 @@ __device__ __forceinline__ void put(const ScaledArgs& p, size_t i, float h) {
   if (p.h32 != nullptr) p.h32[i] = h;
 }
 
-template <int THREADS, int EPT>
+// AT, BT: the terms' types (no choice by a flag inside the loops: every array's loads of a row stand together, under
+// one test that is the same for the whole launch, so that they are all on their way before the first is used)
+template <int THREADS, int EPT, typename AT, typename BT>
 __global__ __launch_bounds__(THREADS) void scaled_add_norm_kernel(ScaledArgs p) {
   __shared__ float red[THREADS / 64];
   const size_t base = (size_t)blockIdx.x * p.D;
   const int D = p.D;
-  float v[EPT];
+  const AT* __restrict__ pa = (const AT*)p.a;
+  const BT* __restrict__ pb = (const BT*)p.b;
+  float v[EPT], t[EPT];
 #pragma unroll
   for (int i = 0; i < EPT; ++i) {
     const int d = threadIdx.x + THREADS * i;
-    v[i] = d < D ? updated(p, base, d) : 0.f;
+    v[i] = d < D ? p.x[base + d] : 0.f;
+    t[i] = 0.f;
   }
-  if (p.a != nullptr) {
+  if (pa != nullptr) {
+    if (p.a_inv != nullptr) {  // (the pieces of an expert sum, added up in their order from zero)
+      const int* rows = p.a_inv + (size_t)blockIdx.x * p.a_k;
+      for (int j = 0; j < p.a_k; ++j) {
+        const size_t at = (size_t)rows[j] * D;
+#pragma unroll
+        for (int i = 0; i < EPT; ++i) {
+          const int d = threadIdx.x + THREADS * i;
+          if (d < D) t[i] += Num<AT>::load(pa + at + d);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) {
+        const int d = threadIdx.x + THREADS * i;
+        if (d < D) t[i] = Num<AT>::load(pa + base + d);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) t[i] *= p.fa;
+    if (pb != nullptr) {
+      float u[EPT];
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) {
+        const int d = threadIdx.x + THREADS * i;
+        u[i] = d < D ? Num<BT>::load(pb + base + d) : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) t[i] = __builtin_fmaf(p.fb, u[i], t[i]);
+    }
+    if (p.vec != nullptr) {
+      float u[EPT];
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) {
+        const int d = threadIdx.x + THREADS * i;
+        u[i] = d < D ? p.vec[d] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) v[i] = __builtin_fmaf(u[i], t[i], v[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) v[i] += t[i];
+    }
 #pragma unroll
     for (int i = 0; i < EPT; ++i) {
       const int d = threadIdx.x + THREADS * i;
@@ -73,6 +142,12 @@ __global__ __launch_bounds__(THREADS) void scaled_add_norm_kernel(ScaledArgs p) 
     }
   }
   if (p.h == nullptr) return;
+  float w[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {  // (asked for before the statistics are there)
+    const int d = threadIdx.x + THREADS * i;
+    w[i] = (p.w != nullptr && d < D) ? p.w[d] : 1.f;
+  }
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < EPT; ++i) ss = __builtin_fmaf(v[i], v[i], ss);
@@ -82,7 +157,7 @@ __global__ __launch_bounds__(THREADS) void scaled_add_norm_kernel(ScaledArgs p) 
     const int d = threadIdx.x + THREADS * i;
     if (d < D) {
       const float h = v[i] * inv;
-      put(p, base + d, p.w != nullptr ? h * p.w[d] : h);
+      put(p, base + d, p.w != nullptr ? h * w[i] : h);
     }
   }
 }
@@ -93,8 +168,9 @@ __global__ __launch_bounds__(THREADS) void scaled_add_norm_wide_kernel(ScaledArg
   const size_t base = (size_t)blockIdx.x * p.D;
   const int D = p.D;
   float ss = 0.f;
+  const Pieces pc = pieces_of(p, blockIdx.x);
   for (int d = threadIdx.x; d < D; d += THREADS) {
-    const float v = updated(p, base, d);
+    const float v = updated(p, pc, base, d);
     p.x[base + d] = v;
     ss = __builtin_fmaf(v, v, ss);
   }
@@ -118,17 +194,22 @@ JLE_API int jle_scaled_add_norm(float* x, const void* a, int a_kind, float fa, c
       (b != nullptr && a == nullptr) || (h == nullptr && h32 != nullptr) || (a_inv != nullptr && (a == nullptr || a_k < 1)))
     return JLE_BAD_ARG;
   ScaledArgs p{x, a, b, vec, w, h, h32, fa, fb, eps, a_kind == 1, b_kind == 1, h_bf16, D, a_inv, a_k};
-  // (which kernel: by the width alone, never by the step's size)
-  if (D <= 256)
-    hipLaunchKernelGGL((scaled_add_norm_kernel<64, 4>), dim3(N), dim3(64), 0, s, p);
-  else if (D <= 1024)
-    hipLaunchKernelGGL((scaled_add_norm_kernel<256, 4>), dim3(N), dim3(256), 0, s, p);
-  else if (D <= 4096)
-    hipLaunchKernelGGL((scaled_add_norm_kernel<256, 16>), dim3(N), dim3(256), 0, s, p);
-  else if (D <= 8192)
-    hipLaunchKernelGGL((scaled_add_norm_kernel<512, 16>), dim3(N), dim3(512), 0, s, p);
-  else
-    hipLaunchKernelGGL((scaled_add_norm_wide_kernel<512>), dim3(N), dim3(512), 0, s, p);
+  // (which kernel: by the width and the terms' types alone, never by the step's size)
+#define JLE_SCALED(AT, BT)                                                                                \
+  do {                                                                                                    \
+    if (D <= 256) hipLaunchKernelGGL((scaled_add_norm_kernel<64, 4, AT, BT>), dim3(N), dim3(64), 0, s, p);  \
+    else if (D <= 1024) hipLaunchKernelGGL((scaled_add_norm_kernel<256, 4, AT, BT>), dim3(N), dim3(256), 0, s, p); \
+    else if (D <= 2048) hipLaunchKernelGGL((scaled_add_norm_kernel<256, 8, AT, BT>), dim3(N), dim3(256), 0, s, p); \
+    else if (D <= 4096) hipLaunchKernelGGL((scaled_add_norm_kernel<256, 16, AT, BT>), dim3(N), dim3(256), 0, s, p); \
+    else if (D <= 8192) hipLaunchKernelGGL((scaled_add_norm_kernel<512, 16, AT, BT>), dim3(N), dim3(512), 0, s, p); \
+    else hipLaunchKernelGGL((scaled_add_norm_wide_kernel<512>), dim3(N), dim3(512), 0, s, p);             \
+  } while (0)
+  const bool a16 = a_kind == 1, b16 = b_kind == 1;
+  if (a16 && (b16 || b == nullptr)) JLE_SCALED(bf16_t, bf16_t);
+  else if (a16) JLE_SCALED(bf16_t, float);
+  else if (b16) JLE_SCALED(float, bf16_t);
+  else JLE_SCALED(float, float);
+#undef JLE_SCALED
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -1,8 +1,13 @@
 """The Sudilorn design in the engine against its plain implementation (``plain_sudilorn.py``): every mechanism alone,
 then whole models however the requests are cut and batched, on the plain ops (CPU) and on the HIP kernels (GPU)."""
 import collections
-import math
+import json
+import os
+import subprocess
+import sys
 import types
+
+import numpy as np
 
 import pytest
 import torch
@@ -203,6 +208,21 @@ def test_delta_rule_long_decoding_through_both_halves_of_its_state(folders, devi
     for sizes in ([T], [3] + [1] * (T - 3), [149, 2, 149]):
         got = _mixer_alone(folders[name], device, layer, sizes, x)
         assert torch.allclose(got, want, rtol=5e-4, atol=5e-5), (got - want).abs().max()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,layer", [("SA", 0), ("SS", 0)])
+def test_delta_rule_prompts_that_end_before_at_and_behind_a_blocks_edge(folders, device, name, layer):
+    """The scan brings a segment's tokens into shared memory 16 at a time, and whole blocks and a segment's last tokens
+    take different stretches of its code: prompts and portions of 15, 16, 17, 31, 32, 33 ... tokens, a portion that
+    starts inside a block, large inputs (decays at both ends)."""
+    cfg, w = P.load(folders[name])
+    for T in (15, 16, 17, 31, 32, 33, 48, 70):
+        x = torch.randn(T, cfg["width"], generator=torch.Generator().manual_seed(T)) * 2.0
+        want = _plain_mixer(cfg, w, layer, x)
+        for sizes in ([T], [5, T - 5], [T - 1, 1]):
+            got = _mixer_alone(folders[name], device, layer, sizes, x)
+            assert torch.allclose(got, want, rtol=5e-4, atol=5e-5), (T, sizes, (got - want).abs().max())
 
 
 def _sharpen_left(mixer):
@@ -508,6 +528,35 @@ def test_greedy_generation_through_the_engine(folders, device):
                     **({"reference_ops": True} if device == "cpu" else {}))
     got = engine.generate(prompts, SamplingParams(max_decode_length=steps))
     assert got == want
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32"])
+def test_trace_run_program(folders_bf16, tmp_path, dtype):
+    """``bin/trace_run`` as a program, on a folder that holds config.json and bfloat16 weights (in float32: in
+    bfloat16 a router's close call may fall the other way, and a program's output says nothing of its choices)."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = folders_bf16["SA"]
+    reqs = traces.random_requests(300, [40, 9, 70, 21, 33], seed=11)
+    steps = traces.mixed(reqs)
+    out_dir = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out_dir), "--max-tokens", str(traces.max_live_tokens(steps)),
+                           "--max-requests", "4"],
+                          input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [ln for ln in proc.stdout.splitlines() if ln.startswith("done")] == [f"done {s['step']}" for s in steps]
+    ref = {rid: _plain_logits(folder, toks) for rid, toks in reqs.items()}
+    at = {rid: 0 for rid in reqs}
+    for s in steps:
+        got = np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4").reshape(-1, 300)
+        o = 0
+        for e in s["entries"]:
+            for wnt in e["want"]:
+                r = ref[e["id"]][at[e["id"]] + wnt]
+                assert float((torch.from_numpy(got[o].copy()) - r).abs().max() / ref[e["id"]].abs().max()) < TOL[dtype]
+                o += 1
+            at[e["id"]] += len(e["tokens"])
 
 
 # ---------------------------------------------------------------------------------------------- configuration
