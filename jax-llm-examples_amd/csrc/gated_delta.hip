@@ -21,8 +21,8 @@ __global__ __launch_bounds__(64) void gdr_prepare_kernel(const T* __restrict__ r
                                                          const float* __restrict__ a_log,
                                                          const float* __restrict__ dt_bias, float* __restrict__ qn,
                                                          float* __restrict__ kn, float* __restrict__ beta,
-                                                         float* __restrict__ decay, float floor, int H, int G, int dk,
-                                                         int dv, int dkp) {
+                                                         float* __restrict__ decay, float* __restrict__ kq,
+                                                         float floor, int H, int G, int dk, int dv, int dkp) {
   const int n = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
   const int C = 2 * G * dk + H * dv;
   if (g == G) {  // the write strengths and decays of the token's heads
@@ -46,6 +46,13 @@ __global__ __launch_bounds__(64) void gdr_prepare_kernel(const T* __restrict__ r
     if (which == 0) inv *= 1.0f / sqrtf((float)dk);
     for (int e = lane; e < dkp; e += 64) dst[e] = e < dk ? Num<T>::load(src + e) * inv : 0.f;
   }
+  // the product of the token's own two unit vectors (what its write adds to its own read-out)
+  const float* qd = qn + ((size_t)n * G + g) * dkp;
+  const float* kd = kn + ((size_t)n * G + g) * dkp;
+  float d = 0.f;
+  for (int e = lane; e < dk; e += 64) d = __builtin_fmaf(qd[e], kd[e], d);  // (this lane's own stores)
+  d = wave_sum(d);
+  if (lane == 0) kq[(size_t)n * G + g] = d;
 }
 
 // KS lanes share a column, each with R consecutive rows of it (KS * R = dkp >= dk, the unit vectors' rows padded with
@@ -80,7 +87,8 @@ struct ScanShape {
 template <typename T, int KS, int R>
 __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows, const float* __restrict__ qn,
                                                       const float* __restrict__ kn, const float* __restrict__ beta,
-                                                      const float* __restrict__ decay, float* __restrict__ state,
+                                                      const float* __restrict__ decay, const float* __restrict__ kq,
+                                                      float* __restrict__ state,
                                                       const int* __restrict__ cu_seqlens,
                                                       const int* __restrict__ state_slots,
                                                       const int* __restrict__ state_phase, float* __restrict__ o_raw,
@@ -88,7 +96,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   using Shape = ScanShape<KS, R>;
   constexpr int TB = Shape::kTB, DKP = Shape::kDkp, NV = Shape::kVecs, cols = 64 / KS;
   __shared__ f32x4 sk[TB * DKP / 4], sq[TB * DKP / 4];
-  __shared__ float sb[TB], sg[TB];
+  __shared__ float sb[TB], sg[TB], skq[TB];
   const int seg = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int ks = lane % KS, c = blockIdx.z * cols + lane / KS;  // (a column's lanes are neighbours)
   const bool live = c < dv;
@@ -124,7 +132,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   f32x4 stk[NV], stq[NV];
 #pragma unroll
   for (int j = 0; j < NV; ++j) stk[j] = stq[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float vnext[TB], vcur[TB], bnext = 0.f, gnext = 1.f;
+  float vnext[TB], vcur[TB], bnext = 0.f, gnext = 1.f, kqnext = 0.f;
   auto ask = [&](int tb) __attribute__((always_inline)) {  // the TB tokens from tb on (those beyond the segment's end: its last token again, unused)
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -143,6 +151,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
       const size_t at = (size_t)min(tb + lane, t1 - 1) * H + h;
       bnext = tb + lane < t1 ? beta[at] : 0.f;
       gnext = tb + lane < t1 ? decay[at] : 1.f;
+      kqnext = kq[(size_t)min(tb + lane, t1 - 1) * G + g];
     }
   };
   auto put = [&]() __attribute__((always_inline)) {
@@ -157,6 +166,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
     if (lane < TB) {
       sb[lane] = bnext;
       sg[lane] = gnext;
+      skq[lane] = kqnext;
     }
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) vcur[tt] = vnext[tt];
@@ -175,22 +185,22 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
         kc[i] = a.x; kc[i + 1] = a.y; kc[i + 2] = a.z; kc[i + 3] = a.w;
         qc[i] = b.x; qc[i + 1] = b.y; qc[i + 2] = b.z; qc[i + 3] = b.w;
       }
-      const float gc = sg[tt], bc = sb[tt];
-      float d4[4] = {0.f, 0.f, 0.f, 0.f};  // (four sums side by side: no chain of R dependent operations)
+      // With S the memory before the token: the write is u = beta (v - g S^T k), the read-out S'^T q of the memory
+      // after it, S' = g S + k u^T, is g S^T q + (k . q) u: both products with S stand side by side, and from one
+      // token to the next leads one multiply-add of the memory.
+      const float gc = sg[tt], bc = sb[tt], kqc = skq[tt];
+      float d4[4] = {0.f, 0.f, 0.f, 0.f}, o4[4] = {0.f, 0.f, 0.f, 0.f};  // (four sums side by side, not a chain of R)
 #pragma unroll
       for (int i = 0; i < R; ++i) {
-        S[i] *= gc;
         d4[i & 3] = __builtin_fmaf(S[i], kc[i], d4[i & 3]);
-      }
-      const float dot = column_lanes_sum<KS>((d4[0] + d4[1]) + (d4[2] + d4[3]));
-      const float u = bc * (vcur[tt] - dot);
-      float o4[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int i = 0; i < R; ++i) {
-        S[i] = __builtin_fmaf(kc[i], u, S[i]);
         o4[i & 3] = __builtin_fmaf(S[i], qc[i], o4[i & 3]);
       }
-      const float out = column_lanes_sum<KS>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+      const float dot = column_lanes_sum<KS>((d4[0] + d4[1]) + (d4[2] + d4[3]));
+      const float oq = column_lanes_sum<KS>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+      const float u = bc * (vcur[tt] - gc * dot);
+      const float out = __builtin_fmaf(kqc, u, gc * oq);
+#pragma unroll
+      for (int i = 0; i < R; ++i) S[i] = __builtin_fmaf(kc[i], u, gc * S[i]);
       if (live && ks == 0 && tb + tt < t1) o_raw[((size_t)(tb + tt) * H + h) * dv + c] = out;
     };
     if (tb + TB <= t1) {  // a whole block: no branch around a token, one stretch of code that the compiler may interleave
@@ -240,8 +250,8 @@ __global__ __launch_bounds__(64) void gdr_out_kernel(const float* __restrict__ o
 template <typename T>
 int launch_gdr(const T* rows, const float* gates, const float* a_log, const float* dt_bias, const float* norm_w,
                const T* gate, float* state, const int* cu_seqlens, const int* state_slots, const int* state_phase,
-               float* qn, float* kn, float* beta, float* decay, float* o_raw, T* out, int N, int R_, int H, int G, int dk,
-               int dv, int dkp, float eps, float floor, hipStream_t s) {
+               float* qn, float* kn, float* beta, float* decay, float* kq, float* o_raw, T* out, int N, int R_, int H,
+               int G, int dk, int dv, int dkp, float eps, float floor, hipStream_t s) {
   // lanes a column: the fewest that leave a lane at most 16 rows of it (by the sizes alone)
   int KS = 1;
   while (KS < 64 && (dk + KS - 1) / KS > 16) KS <<= 1;
@@ -249,7 +259,7 @@ int launch_gdr(const T* rows, const float* gates, const float* a_log, const floa
   const int RR = per <= 4 ? 4 : per <= 8 ? 8 : per <= 16 ? 16 : 32;
   if (dkp != KS * RR) return JLE_BAD_ARG;
   hipLaunchKernelGGL(gdr_prepare_kernel<T>, dim3(N, G + 1), dim3(64), 0, s, rows, gates, a_log, dt_bias, qn, kn, beta,
-                     decay, floor, H, G, dk, dv, dkp);
+                     decay, kq, floor, H, G, dk, dv, dkp);
   JLE_LAUNCH_CHECK();
   // A step with few (segment, head) pairs leaves most of the machine idle, and what a token takes is the length of its
   // chain of dependent operations: then a column gets more lanes with fewer rows each (the row's width stays).
@@ -261,7 +271,7 @@ int launch_gdr(const T* rows, const float* gates, const float* a_log, const floa
   const int cols_ = 64 / ks;
   const dim3 grid(R_, H, (dv + cols_ - 1) / cols_);
 #define JLE_SCAN(KS_, RR_)                                                                                          \
-  hipLaunchKernelGGL((gdr_scan_kernel<T, KS_, RR_>), grid, dim3(64), 0, s, rows, qn, kn, beta, decay, state, cu_seqlens, \
+  hipLaunchKernelGGL((gdr_scan_kernel<T, KS_, RR_>), grid, dim3(64), 0, s, rows, qn, kn, beta, decay, kq, state, cu_seqlens, \
                      state_slots, state_phase, o_raw, H, G, dk, dv)
 #define JLE_SCAN_R(KS_)              \
   do {                               \
@@ -305,8 +315,8 @@ JLE_API int jle_gated_delta_padded(int dk) {
 JLE_API int jle_gated_delta(const void* rows, int is_bf16, const float* gates, const float* a_log, const float* dt_bias,
                             const float* norm_w, const void* gate, float* state, const int* cu_seqlens,
                             const int* state_slots, const int* state_phase, float* qn, float* kn, float* beta,
-                            float* decay, float* o_raw, void* out, int N, int R, int H, int G, int dk, int dv, float eps,
-                            float floor, hipStream_t s) {
+                            float* decay, float* kq, float* o_raw, void* out, int N, int R, int H, int G, int dk, int dv,
+                            float eps, float floor, hipStream_t s) {
   if (N <= 0) return 0;
   const int dkp = jle_gated_delta_padded(dk);
   if (dkp <= 0 || ((uintptr_t)qn | (uintptr_t)kn) % 16) return JLE_BAD_ARG;
@@ -315,9 +325,9 @@ JLE_API int jle_gated_delta(const void* rows, int is_bf16, const float* gates, c
     return JLE_BAD_ARG;
   if (is_bf16)
     return launch_gdr<bf16_t>((const bf16_t*)rows, gates, a_log, dt_bias, norm_w, (const bf16_t*)gate, state, cu_seqlens,
-                              state_slots, state_phase, qn, kn, beta, decay, o_raw, (bf16_t*)out, N, R, H, G, dk, dv, dkp,
+                              state_slots, state_phase, qn, kn, beta, decay, kq, o_raw, (bf16_t*)out, N, R, H, G, dk, dv, dkp,
                               eps, floor, s);
   return launch_gdr<float>((const float*)rows, gates, a_log, dt_bias, norm_w, (const float*)gate, state, cu_seqlens,
-                           state_slots, state_phase, qn, kn, beta, decay, o_raw, (float*)out, N, R, H, G, dk, dv, dkp, eps,
+                           state_slots, state_phase, qn, kn, beta, decay, kq, o_raw, (float*)out, N, R, H, G, dk, dv, dkp, eps,
                            floor, s);
 }

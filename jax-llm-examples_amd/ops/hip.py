@@ -93,8 +93,8 @@ _SIGNATURES = {
     "jle_heads_prepare": [_vp, _vp, _vp, _vp, _i, _i, _f, _f, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i,
                           _vp],
     "jle_diff_combine": [_vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_gated_delta": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
-                        _i, _i, _i, _f, _f, _vp],
+    "jle_gated_delta": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
+                        _i, _i, _i, _i, _f, _f, _vp],
     "jle_moe_choose": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_relu2": [_vp, _vp, _i, _ll, _vp],
     "jle_conv_rows_act": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
@@ -924,14 +924,16 @@ class HipOps:
         dkp = self._query("jle_gated_delta_padded", dk)  # (the unit vectors' rows, filled up to what the scan's lanes hold)
         if dkp < dk:
             raise KernelError(f"the gated delta rule's kernels take keys of up to 2048 elements, not {dk}")
-        scratch = torch.empty(n * (2 * G * dkp + 2 * H + H * dv), dtype=torch.float32, device=dev)
+        scratch = torch.empty(n * (2 * G * dkp + 2 * H + G + H * dv), dtype=torch.float32, device=dev)
         qn, kn = scratch[: n * G * dkp], scratch[n * G * dkp: 2 * n * G * dkp]
         o = 2 * n * G * dkp
-        beta, decay, o_raw = scratch[o: o + n * H], scratch[o + n * H: o + 2 * n * H], scratch[o + 2 * n * H:]
+        beta, decay, kq = scratch[o: o + n * H], scratch[o + n * H: o + 2 * n * H], scratch[o + 2 * n * H: o + 2 * n * H + n * G]
+        o_raw = scratch[o + 2 * n * H + n * G:]
         out = torch.empty(n, H * dv, dtype=rows.dtype, device=dev)
         self._call("jle_gated_delta", _p(rows), self._is_bf16(rows), _p(gates), _p(a_log), _p(dt_bias), _p(norm_weight),
                    _p(out_gate), _p(state), _p(ctx.cu_seqlens), _p(ctx.state_slots), _p(ctx.state_phase), _p(qn), _p(kn),
-                   _p(beta), _p(decay), _p(o_raw), _p(out), n, ctx.num_segments, H, G, dk, dv, float(eps), float(floor))
+                   _p(beta), _p(decay), _p(kq), _p(o_raw), _p(out), n, ctx.num_segments, H, G, dk, dv, float(eps),
+                   float(floor))
         return out
 
     def conv_qk_prepare(self, proj, bias, conv_w, taps: int, state, num_heads: int, num_kv_heads: int, head_dim: int,
