@@ -93,17 +93,17 @@ def design_configs(size: dict, layers: int):
     # of attention with two score maps per head (half the heads, values twice as wide), and so on; eight scored
     # experts in four groups, two a token; its closest model here is the same Llama 4 with routed layers
     s_left = {"heads": size["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-              "mask": {"size": size["span"], "keep_first": 4}, "rot": {"base": 500000.0, "dims": 64}}
+              "mask": {"size": size["span"], "keep_first": 8}, "rot": {"base": 10000.0, "dims": 64}}
     s_right = {"heads": size["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "conv": 4}
-    s_diff = {"heads": size["heads"] // 2, "kv_heads": 4, "dim": 128, "vdim": 256, "scale": 128 ** -0.5, "diff": 0.6,
+    s_diff = {"heads": size["heads"] // 2, "kv_heads": 4, "dim": 128, "vdim": 256, "scale": 128 ** -0.5, "diff": 0.5,
               "conv": 4, "mask": {"size": size["span"]}, "rot": {"base": 500000.0, "dims": 64, "scaling": yarn}}
     s_moe = {"kind": "moe", "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}},
              "expert": {"ff": size["ff"] // 2}}
     sudilorn = {"architecture": "Sudilorn", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-5},
-                "residual_mult": 0.5,
+                "residual_mult": 0.7,
                 "layers": [{"type": "attention", "mixer": s_diff, "mlp": s_moe} if i % 3 == 2 else
-                           {"type": "parallel", "mixer": {"left": s_left, "right": s_right, "left_scale": 0.8,
-                                                          "right_scale": 0.5}, "mlp": s_moe} for i in range(layers)]}
+                           {"type": "parallel", "mixer": {"left": s_left, "right": s_right, "left_scale": 1.0,
+                                                          "right_scale": 0.7}, "mlp": s_moe} for i in range(layers)]}
     return {"rovidra": rovidra, "tiradra": tiradra, "llama4-dense": llama, "mazotar": mazotar, "llama4-moe": llama_moe,
             "sudilorn": sudilorn}
 

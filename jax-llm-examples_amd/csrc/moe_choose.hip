@@ -17,21 +17,27 @@ __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict_
                                                         const float* __restrict__ correction, int* __restrict__ ids,
                                                         float* __restrict__ weights, int N, int E, int top_k,
                                                         int groups, int keep, int terms) {
+  // (a thread's lists lie in shared memory: indexed by values that are known only when the kernel runs, they would
+  // otherwise be kept in scratch memory)
+  __shared__ float score_all[kMaxGroups][64];
+  __shared__ int chosen_all[kMaxTop][64];
   const int n = blockIdx.x * 64 + threadIdx.x;
   if (n >= N) return;
+  const int me = threadIdx.x;
   const float* z = logits + (size_t)n * E;
   auto choice = [&](int e) { return sigmoidf_(z[e]) + (correction != nullptr ? correction[e] : 0.f); };
   unsigned long long kept = ~0ull;  // bit gi: group gi's experts can be chosen
   const int per = groups > 0 ? E / groups : E;
   if (groups > 0) {
-    float score[kMaxGroups];
     for (int gi = 0; gi < groups; ++gi) {
       float best[kMaxTerms];
+#pragma unroll
       for (int i = 0; i < kMaxTerms; ++i) best[i] = -INFINITY;
       for (int e = gi * per; e < (gi + 1) * per; ++e) {
         float c = choice(e);
-        for (int i = 0; i < terms; ++i) {  // (kept in descending order)
-          if (c > best[i]) {
+#pragma unroll
+        for (int i = 0; i < kMaxTerms; ++i) {  // (kept in descending order)
+          if (i < terms && c > best[i]) {
             const float t = best[i];
             best[i] = c;
             c = t;
@@ -39,8 +45,10 @@ __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict_
         }
       }
       float sum = 0.f;
-      for (int i = 0; i < terms && i < per; ++i) sum += best[i];
-      score[gi] = sum;
+#pragma unroll
+      for (int i = 0; i < kMaxTerms; ++i)
+        if (i < terms && i < per) sum += best[i];
+      score_all[gi][me] = sum;
     }
     kept = 0ull;
     for (int r = 0; r < keep; ++r) {
@@ -48,22 +56,22 @@ __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict_
       float top = 0.f;
       for (int gi = 0; gi < groups; ++gi) {
         if ((kept >> gi) & 1ull) continue;
-        if (at < 0 || score[gi] > top) {
+        const float sc = score_all[gi][me];
+        if (at < 0 || sc > top) {
           at = gi;
-          top = score[gi];
+          top = sc;
         }
       }
       kept |= 1ull << at;
     }
   }
-  int chosen[kMaxTop];
   for (int r = 0; r < top_k; ++r) {
     int at = -1;
     float top = 0.f;
     for (int e = 0; e < E; ++e) {
       if (groups > 0 && !((kept >> (e / per)) & 1ull)) continue;
       bool taken = false;
-      for (int i = 0; i < r; ++i) taken |= chosen[i] == e;
+      for (int i = 0; i < r; ++i) taken |= chosen_all[i][me] == e;
       if (taken) continue;
       const float c = choice(e);
       if (at < 0 || c > top) {
@@ -71,7 +79,7 @@ __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict_
         top = c;
       }
     }
-    chosen[r] = at;
+    chosen_all[r][me] = at;
     ids[(size_t)n * top_k + r] = at;
     weights[(size_t)n * top_k + r] = sigmoidf_(z[at]);
   }

@@ -84,7 +84,7 @@ def test_branch_outputs_with_factors_and_the_next_norm(device, width):
 def test_stretched_rates_of_half_split_pairs():
     """The position part's rates and magnitude are the plain formula's, with ramps that start before the first pair,
     end beyond the last, or have no width."""
-    for base, dims, sc in ((250000.0, 32, (4.0, 2048, 32.0, 1.0)), (5000.0, 12, (8.0, 64, 4.0, 1.0)),
+    for base, dims, sc in ((100000.0, 48, (4.0, 4096, 16.0, 1.0)), (5000.0, 12, (8.0, 64, 4.0, 1.0)),
                            (30.0, 6, (4.0, 16, 8.0, 2.0)), (10000.0, 8, (2.0, 32, 2.0, 2.0)), (100.0, 8, None)):
         rot = {"base": base, "dims": dims}
         if sc is not None:
