@@ -9,7 +9,7 @@ using namespace jle;
 
 namespace {
 
-constexpr int kMaxGroups = 64, kMaxTerms = 4, kMaxTop = 16;
+constexpr int kMaxGroups = 64, kMaxTerms = 4, kMaxTop = 16, kCached = 64;
 
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 
@@ -25,7 +25,15 @@ __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict_
   if (n >= N) return;
   const int me = threadIdx.x;
   const float* z = logits + (size_t)n * E;
-  auto choice = [&](int e) { return sigmoidf_(z[e]) + (correction != nullptr ? correction[e] : 0.f); };
+  // the choice scores of up to kCached experts are formed once and kept in shared memory (a thread walks through them
+  // top_k + 1 times); with more experts they are formed anew each time
+  __shared__ float cached[kCached][64];
+  const bool in_lds = E <= kCached;
+  if (in_lds)
+    for (int e = 0; e < E; ++e) cached[e][me] = sigmoidf_(z[e]) + (correction != nullptr ? correction[e] : 0.f);
+  auto choice = [&](int e) {
+    return in_lds ? cached[e][me] : sigmoidf_(z[e]) + (correction != nullptr ? correction[e] : 0.f);
+  };
   unsigned long long kept = ~0ull;  // bit gi: group gi's experts can be chosen
   const int per = groups > 0 ? E / groups : E;
   if (groups > 0) {
