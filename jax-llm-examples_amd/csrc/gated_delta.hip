@@ -96,7 +96,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   using Shape = ScanShape<KS, R>;
   constexpr int TB = Shape::kTB, DKP = Shape::kDkp, NV = Shape::kVecs, cols = 64 / KS;
   __shared__ f32x4 sk[TB * DKP / 4], sq[TB * DKP / 4];
-  __shared__ float sb[TB], sg[TB], skq[TB];
+  __shared__ f32x4 ssc[TB];  // a token's decay, write strength and k . q together: one trip to shared memory
   const int seg = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int ks = lane % KS, c = blockIdx.z * cols + lane / KS;  // (a column's lanes are neighbours)
   const bool live = c < dv;
@@ -164,9 +164,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
       }
     }
     if (lane < TB) {
-      sb[lane] = bnext;
-      sg[lane] = gnext;
-      skq[lane] = kqnext;
+      ssc[lane] = f32x4{gnext, bnext, kqnext, 0.f};
     }
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) vcur[tt] = vnext[tt];
@@ -177,6 +175,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
   for (int tb = t0; tb < t1; tb += TB) {
     const bool more = tb + TB < t1;
     if (more) ask(tb + TB);
+    float outs[TB];  // (the block's read-outs: stored together behind its last token)
     auto token = [&](int tt) __attribute__((always_inline)) {
       float kc[R], qc[R];
 #pragma unroll
@@ -188,7 +187,8 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
       // With S the memory before the token: the write is u = beta (v - g S^T k), the read-out S'^T q of the memory
       // after it, S' = g S + k u^T, is g S^T q + (k . q) u: both products with S stand side by side, and from one
       // token to the next leads one multiply-add of the memory.
-      const float gc = sg[tt], bc = sb[tt], kqc = skq[tt];
+      const f32x4 sc = ssc[tt];
+      const float gc = sc.x, bc = sc.y, kqc = sc.z;
       float d4[4] = {0.f, 0.f, 0.f, 0.f}, o4[4] = {0.f, 0.f, 0.f, 0.f};  // (four sums side by side, not a chain of R)
 #pragma unroll
       for (int i = 0; i < R; ++i) {
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
       const float out = __builtin_fmaf(kqc, u, gc * oq);
 #pragma unroll
       for (int i = 0; i < R; ++i) S[i] = __builtin_fmaf(kc[i], u, gc * S[i]);
-      if (live && ks == 0 && tb + tt < t1) o_raw[((size_t)(tb + tt) * H + h) * dv + c] = out;
+      outs[tt] = out;
     };
     if (tb + TB <= t1) {  // a whole block: no branch around a token, one stretch of code that the compiler may interleave
 #pragma unroll
@@ -210,6 +210,12 @@ __global__ __launch_bounds__(64) void gdr_scan_kernel(const T* __restrict__ rows
 #pragma unroll
       for (int tt = 0; tt < TB; ++tt)
         if (tb + tt < t1) token(tt);
+    }
+    if (live && ks == 0) {
+      float* op = o_raw + ((size_t)tb * H + h) * dv + c;
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt)
+        if (tb + tt < t1) op[(size_t)tt * H * dv] = outs[tt];
     }
     __syncthreads();
     if (more) put();
